@@ -170,6 +170,9 @@ def load_hf_config(model: str, overrides: Optional[dict] = None) -> HFConfig:
     if d.get("architecture") == "Rapovik":         # likewise, with a loop over part of the layers
         from .models.rapovik import normalise_config as rapovik_config
         d = rapovik_config(d, model if os.path.isdir(model) else None)
+    if d.get("architecture") == "Sevazen":         # a layer list of attention variants; layers may share weights
+        from .models.sevazen import normalise_config as sevazen_config
+        d = sevazen_config(d, model if os.path.isdir(model) else None)
     if d.get("model_type") in ("exaone", "telechat", "qwen", "chatglm"):
         from .models.renamed_decoders import normalise_config
         d = normalise_config(d)
@@ -337,7 +340,7 @@ class ModelConfig:
                          # encoder-decoder: the cross-attention cache is per-request state of the same kind
                          "WhisperForConditionalGeneration", "BartForConditionalGeneration", "BartModel",
                          "MllamaForConditionalGeneration", "Zamba2ForCausalLM", "Plamo2ForCausalLM",
-                         "Florence2ForConditionalGeneration", "NositarForCausalLM", "RapovikForCausalLM")
+                         "Florence2ForConditionalGeneration", "NositarForCausalLM", "RapovikForCausalLM", "SevazenForCausalLM")
                    for a in self.architectures)
 
     @property

@@ -63,7 +63,8 @@ def grouped_topk(scores: torch.Tensor, k: int, renormalize: bool, num_expert_gro
 
 class UnquantizedMoEMethod:
     def create_weights(self, layer: "FusedMoE", E: int, H: int, I: int, dtype: torch.dtype) -> None:
-        w13 = nn.Parameter(torch.empty(E, 2 * I, H, dtype=dtype), requires_grad=False)
+        w13 = nn.Parameter(torch.empty(E, (2 if getattr(layer, "gated", True) else 1) * I, H, dtype=dtype),
+                           requires_grad=False)
         w2 = nn.Parameter(torch.empty(E, H, I, dtype=dtype), requires_grad=False)
         layer.register_parameter("w13_weight", w13)
         layer.register_parameter("w2_weight", w2)
@@ -76,7 +77,7 @@ class UnquantizedMoEMethod:
     def apply(self, layer: "FusedMoE", x: torch.Tensor, topk_w: torch.Tensor, topk_ids: torch.Tensor) -> torch.Tensor:
         return ops.fused_moe(x, layer.w13_weight, layer.w2_weight, topk_w, topk_ids,
                              activation=getattr(layer, "activation", "silu"),
-                             act_limit=getattr(layer, "act_limit", 0.0))
+                             act_limit=getattr(layer, "act_limit", 0.0), gated=getattr(layer, "gated", True))
 
 
 class FusedMoE(nn.Module):
@@ -88,8 +89,12 @@ class FusedMoE(nn.Module):
                  topk_group: Optional[int] = None, quant_config=None, prefix: str = "",
                  custom_routing_function: Optional[Callable] = None, scoring_func: str = "softmax",
                  e_score_correction_bias: Optional[torch.Tensor] = None, routed_scaling_factor: float = 1.0,
-                 activation: str = "silu", act_limit: float = 0.0):
+                 activation: str = "silu", act_limit: float = 0.0, gated: bool = True):
         super().__init__()
+        # gated=False: experts of the form W2 act(W1 x), no second (up) half; their first weight loads as "w1"
+        self.gated = bool(gated)
+        if not self.gated and quant_config is not None and quant_config.get_quant_method(self, prefix) is not None:
+            raise NotImplementedError(f"{prefix}: quantised experts without a gate half")
         if activation not in ops.MOE_ACTIVATIONS:
             raise ValueError(f"{prefix}: expert activation {activation!r} is not supported "
                              f"(supported: {', '.join(ops.MOE_ACTIVATIONS)})")

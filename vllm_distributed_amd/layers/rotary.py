@@ -31,14 +31,64 @@ def _yarn_range(low_rot, high_rot, dim, base, max_pos) -> tuple[int, int]:
     return max(lo, 0), min(hi, dim - 1)
 
 
-def _ramp(lo: float, hi: float, n: int) -> torch.Tensor:
+def _ramp(lo: float, hi: float, n: int, dtype: torch.dtype = torch.float32) -> torch.Tensor:
     if lo == hi:
         hi += 0.001
-    return ((torch.arange(n, dtype=torch.float32) - lo) / (hi - lo)).clamp(0, 1)
+    return ((torch.arange(n, dtype=dtype) - lo) / (hi - lo)).clamp(0, 1)
 
 
 def yarn_mscale(scale: float = 1.0, mscale: float = 1.0) -> float:
     return 1.0 if scale <= 1 else 0.1 * mscale * math.log(scale) + 1.0
+
+
+def yarn_freqs(inv: torch.Tensor, factor: float, rot_dim: int, base: float, orig_max: int, beta_fast: float = 32,
+               beta_slow: float = 1, extrapolation_factor: float = 1) -> torch.Tensor:
+    """YaRN: frequencies below the ramp keep their value, those above it are divided by ``factor``, linear between."""
+    lo, hi = _yarn_range(beta_fast, beta_slow, rot_dim, base, orig_max)
+    mask = (1 - _ramp(lo, hi, rot_dim // 2, inv.dtype)) * extrapolation_factor
+    return inv / factor * (1 - mask) + inv * mask
+
+
+def llama3_freqs(inv: torch.Tensor, factor: float, low: float, high: float, orig_max: int) -> torch.Tensor:
+    """Llama-3.1: wavelengths under orig_max / high keep their frequency, those over orig_max / low are divided by
+    ``factor``, a linear blend between."""
+    wave = 2 * math.pi / inv
+    smooth = (orig_max / wave - low) / (high - low) if high != low else torch.zeros_like(inv)
+    mid = (1 - smooth) * inv / factor + smooth * inv
+    return torch.where(wave < orig_max / high, inv, torch.where(wave > orig_max / low, inv / factor, mid))
+
+
+_HALF_SPLIT_TABLES: dict = {}
+
+
+def half_split_cos_sin(max_len: int, rot_dim: int, base: float, scaling: Optional[dict], device) -> torch.Tensor:
+    """fp32 [max_len, rot_dim] for kernels that rotate in fp32: cos(p f_i) for i < rot_dim / 2, then sin(p f_i), with
+    f_i = base^(-2i / rot_dim) rescaled by ``scaling``: None, {"kind": "llama3", factor, low, high, original} or
+    {"kind": "yarn", factor, original, fast, slow, magnitude} (cos and sin times ``magnitude``).  Angles are formed in
+    fp64 and rounded once."""
+    sc = dict(scaling or {})
+    key = (int(max_len), int(rot_dim), float(base), tuple(sorted(sc.items())), str(device))
+    t = _HALF_SPLIT_TABLES.get(key)
+    if t is not None:
+        return t
+    if rot_dim <= 0:
+        t = torch.zeros((max_len, 1), dtype=torch.float32, device=device)
+    else:
+        inv = 1.0 / (float(base) ** (torch.arange(0, rot_dim, 2, dtype=torch.float64) / rot_dim))
+        mag = 1.0
+        kind = sc.get("kind")
+        if kind == "llama3":
+            inv = llama3_freqs(inv, float(sc["factor"]), float(sc["low"]), float(sc["high"]), int(sc["original"]))
+        elif kind == "yarn":
+            inv = yarn_freqs(inv, float(sc["factor"]), rot_dim, float(base), int(sc["original"]),
+                             float(sc.get("fast", 32)), float(sc.get("slow", 1)))
+            mag = float(sc.get("magnitude", yarn_mscale(float(sc["factor"]))))
+        elif kind is not None:
+            raise ValueError(f"unknown frequency scaling {kind!r}")
+        ang = torch.outer(torch.arange(max_len, dtype=torch.float64), inv)
+        t = torch.cat((ang.cos() * mag, ang.sin() * mag), dim=-1).float().contiguous().to(device)
+    _HALF_SPLIT_TABLES[key] = t
+    return t
 
 
 class RotaryEmbedding(nn.Module):
@@ -117,11 +167,8 @@ class YaRNScalingRotaryEmbedding(RotaryEmbedding):
         super().__init__(head_size, rotary_dim, int(max_position * factor), base, is_neox_style)
 
     def _freqs(self):
-        extra = _inv_freq(self.base, self.rotary_dim)
-        inter = extra / self.factor
-        lo, hi = _yarn_range(self.beta_fast, self.beta_slow, self.rotary_dim, self.base, self.orig_max)
-        mask = (1 - _ramp(lo, hi, self.rotary_dim // 2)) * self.extrapolation_factor
-        return inter * (1 - mask) + extra * mask
+        return yarn_freqs(_inv_freq(self.base, self.rotary_dim), self.factor, self.rotary_dim, self.base, self.orig_max,
+                          self.beta_fast, self.beta_slow, self.extrapolation_factor)
 
     def _mscale(self):
         return self._m
@@ -134,13 +181,7 @@ class Llama3RotaryEmbedding(RotaryEmbedding):
         super().__init__(head_size, rotary_dim, max_position, base, is_neox_style)
 
     def _freqs(self):
-        inv = _inv_freq(self.base, self.rotary_dim)
-        wave = 2 * math.pi / inv
-        smooth = (self.orig_max / wave - self.low) / (self.high - self.low) if self.high != self.low else \
-            torch.zeros_like(inv)
-        low_w, high_w = self.orig_max / self.low, self.orig_max / self.high
-        mid = (1 - smooth) * inv / self.factor + smooth * inv
-        return torch.where(wave < high_w, inv, torch.where(wave > low_w, inv / self.factor, mid))
+        return llama3_freqs(_inv_freq(self.base, self.rotary_dim), self.factor, self.low, self.high, self.orig_max)
 
 
 class LongRoPEScaledRotaryEmbedding(RotaryEmbedding):

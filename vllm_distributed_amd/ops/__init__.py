@@ -907,7 +907,7 @@ def moe_grouped_ok(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor) -> bool
             and w13.shape[0] <= 1024)
 
 
-EPI_PLAIN, EPI_GATE_UP, EPI_DOWN = 0, 1, 2
+EPI_PLAIN, EPI_GATE_UP, EPI_DOWN, EPI_UP_ACT = 0, 1, 2, 3
 SC_NONE, SC_TOKEN, SC_BLOCK = 0, 1, 2
 
 
@@ -1042,7 +1042,7 @@ def moe_align_tiles(topk_ids: torch.Tensor, E: int, rows_per_tile: int):
 
 
 def _moe_tiled(x, w13, w2, topk_w, topk_ids, w13_scale, w2_scale, block_scales: bool = False,
-               activation: str = "silu", x_scale=None, out_dtype=None, act_limit: float = 0.0):
+               activation: str = "silu", x_scale=None, out_dtype=None, act_limit: float = 0.0, gated: bool = True):
     """Compute-bound batches: both expert GEMMs run as LDS-tiled MFMA GEMMs over the expert-sorted pairs
     (ops/csrc/gemm_tile.hip).  e4m3 weights: activations are quantised per token (or per group of 128
     with block-scaled weights) and the fp8 matrix cores do the products; 16-bit weights: 16-bit MFMA.
@@ -1052,7 +1052,7 @@ def _moe_tiled(x, w13, w2, topk_w, topk_ids, w13_scale, w2_scale, block_scales: 
     T, H = x.shape
     k = topk_ids.shape[1]
     E, I2, _ = w13.shape
-    I = I2 // 2
+    I = I2 // 2 if gated else I2
     P_ = T * k
     dev = x.device
     rows = _tile_rows(P_ / E)
@@ -1076,7 +1076,8 @@ def _moe_tiled(x, w13, w2, topk_w, topk_ids, w13_scale, w2_scale, block_scales: 
         mode, xq, xs = SC_NONE, _contig_last(x), None
     N.call("vda_tile_gemm", inter.data_ptr(), xq.data_ptr(), w13.data_ptr(), N.ptr(xs), N.ptr(w13_scale), None, None,
            sorted_ids.data_ptr(), te.data_ptr(), tb.data_ptr(), tend.data_ptr(), ntl.data_ptr(), 0, I, H, k,
-           max_tiles, xq.stride(0), I, I2 * H, EPI_GATE_UP, mode, rows, N.dt(xq.dtype), N.dt(odt), N.ACT[activation],
+           max_tiles, xq.stride(0), I, I2 * H, EPI_GATE_UP if gated else EPI_UP_ACT, mode, rows, N.dt(xq.dtype),
+           N.dt(odt), N.ACT[activation],
            float(act_limit), st)
     if fp8:
         hq, hs = per_group_fp8_quant(inter) if block_scales else per_token_fp8_quant(inter)
@@ -1103,8 +1104,8 @@ def moe_fp8_rows_ok(w13: torch.Tensor, w2: torch.Tensor, dtype: torch.dtype, pai
                  or not moe_grouped_ok(probe, w13, w2)))
 
 
-def moe_tiled_ok(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor) -> bool:
-    I = w13.shape[1] // 2
+def moe_tiled_ok(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, gated: bool = True) -> bool:
+    I = w13.shape[1] // 2 if gated else w13.shape[1]
     return (x.dtype in (torch.bfloat16, torch.float16) and w13.dtype in (x.dtype, torch.float8_e4m3fn)
             and w13.dtype == w2.dtype and tile_gemm_ok(w13.shape[2], w13.dtype) and tile_gemm_ok(I, w13.dtype)
             and I % 64 == 0 and w2.shape[1] % 4 == 0 and w13.shape[0] <= 1024)
@@ -1133,23 +1134,24 @@ def moe_rows_form(num_pairs: int, num_experts: int, rows: int, weight_bytes: int
     return wide if avg >= 8 and (fills or avg >= 64) else 0
 
 
-def moe_pairs_ok(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor) -> bool:
+def moe_pairs_ok(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, gated: bool = True) -> bool:
     """The plain-arithmetic expert kernel: any widths, weights of the activations' type (16-bit or fp32)."""
     return (x.dtype in (torch.bfloat16, torch.float16, torch.float32) and w13.dtype == x.dtype and w2.dtype == x.dtype
-            and (w13.shape[2] + w13.shape[1] // 2) * 4 <= 60 * 1024 and w13.is_contiguous() and w2.is_contiguous())
+            and (w13.shape[2] + w13.shape[1] // (2 if gated else 1)) * 4 <= 60 * 1024 and w13.is_contiguous()
+            and w2.is_contiguous())
 
 
-def _moe_pairs(x, w13, w2, topk_w, topk_ids, activation: str, act_limit: float):
+def _moe_pairs(x, w13, w2, topk_w, topk_ids, activation: str, act_limit: float, gated: bool = True):
     """Experts of sizes the MFMA kernels are not built for: one workgroup per (token, choice) pair
     (ops/csrc/moe.hip, vda_moe_pairs); sums over a token's choices in a fixed order."""
     T, H = x.shape
     k = topk_ids.shape[1]
-    I, Ho = w13.shape[1] // 2, w2.shape[1]
+    I, Ho = w13.shape[1] // (2 if gated else 1), w2.shape[1]
     out = torch.empty((T, Ho), dtype=x.dtype, device=x.device)
     part = torch.empty((T * k, Ho), dtype=torch.float32, device=x.device)
     N.call("vda_moe_pairs", out.data_ptr(), out.stride(0), part.data_ptr(), x.data_ptr(), x.stride(0), w13.data_ptr(),
            w2.data_ptr(), topk_w.contiguous().data_ptr(), topk_ids.contiguous().data_ptr(), T, H, I, Ho, k,
-           N.ACT[activation], float(act_limit), N.dt(x.dtype), N.stream())
+           N.ACT[activation], float(act_limit), int(gated), N.dt(x.dtype), N.stream())
     return out
 
 
@@ -1159,15 +1161,27 @@ MOE_ACTIVATIONS = ("silu", "gelu", "gelu_tanh", "gelu_pytorch_tanh", "relu", "re
 def fused_moe(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, topk_w: torch.Tensor, topk_ids: torch.Tensor,
               w13_scale: Optional[torch.Tensor] = None, w2_scale: Optional[torch.Tensor] = None,
               block_scales: bool = False, activation: str = "silu", x_scale: Optional[torch.Tensor] = None,
-              out_dtype: Optional[torch.dtype] = None, act_limit: float = 0.0) -> torch.Tensor:
+              out_dtype: Optional[torch.dtype] = None, act_limit: float = 0.0, gated: bool = True) -> torch.Tensor:
     """Routed gated expert MLPs, out[t] = sum_j w[t, j] * W2_e(act(Wg_e x_t) * (Wu_e x_t)) with ``activation`` one of
     MOE_ACTIVATIONS (reference: vllm/model_executor/layers/fused_moe/fused_moe.py:1003,1034 ``activation``), fused
     into the first GEMM's epilogue in every kernel form.  x [T,H]; w13 [E,2I,H] (gate rows then up rows); w2 [E,H,I];
     topk_w f32 [T,k]; topk_ids i32 [T,k] with local expert ids, negative = not on this rank.
     e4m3 weights carry one scale per expert, or with ``block_scales`` one per 128 x 128 block
-    (w13_scale [E, 2I/128, H/128], w2_scale [E, H/128, I/128])."""
+    (w13_scale [E, 2I/128, H/128], w2_scale [E, H/128, I/128]).
+    ``gated=False``: experts without a gate half, out[t] = sum_j w[t, j] * W2_e act(Wu_e x_t) with w13 [E,I,H]; 16-bit or
+    fp32 weights, through the tiled MFMA GEMMs (widths they take) or the per-pair kernel (any widths)."""
     if activation not in MOE_ACTIVATIONS:
         raise ValueError(f"expert activation {activation!r} is not supported (supported: {', '.join(MOE_ACTIVATIONS)})")
+    if not gated:
+        if activation == "clamped_swiglu" or w13_scale is not None or w2_scale is not None or x_scale is not None:
+            raise ValueError("experts without a gate half take an element-wise activation and unquantised weights")
+        if _dev(x) and moe_tiled_ok(x, w13, w2, gated=False):
+            return _moe_tiled(_contig_last(x), w13, w2, topk_w, topk_ids, None, None, False, activation, gated=False)
+        if _dev(x) and moe_pairs_ok(x, w13, w2, gated=False):
+            return _moe_pairs(_contig_last(x), w13, w2, topk_w, topk_ids, activation, 0.0, gated=False)
+        if _dev(x) and torch.cuda.is_current_stream_capturing():
+            raise RuntimeError(f"expert shapes {tuple(w13.shape)} / {tuple(w2.shape)} are outside the expert kernels")
+        return R.fused_moe(x, w13, w2, topk_w, topk_ids, None, None, False, activation, 0.0, gated=False)
     if x_scale is not None:
         # x is e4m3 with one scale per row (see moe_fp8_rows_ok): straight into the fp8 tiles, or widened again
         odt = out_dtype or torch.bfloat16
@@ -1539,4 +1553,87 @@ def mlstm(proj: torch.Tensor, i_bias: torch.Tensor, f_bias: torch.Tensor, norm_w
            i_bias.data_ptr(), f_bias.data_ptr(), norm_w.data_ptr(), state_nm.data_ptr(), state_s.data_ptr(),
            query_start_loc.data_ptr(), seq_lens.data_ptr(), slot_table.data_ptr(), slot_table.stride(0), T,
            seq_lens.shape[0], H, D, Dv, state_nm.shape[2], float(cap), float(eps), N.dt(proj.dtype), N.stream())
+    return out
+
+
+# ---- fp32 residual with a layer norm on every sub-layer's output ------------------------------------------------
+def residual_layer_norm(x: torch.Tensor, y: Optional[torch.Tensor], weight: torch.Tensor,
+                        bias: Optional[torch.Tensor], eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """One pass over the fp32 residual ``x`` [T, W].  With ``y`` (a sub-layer's output): x += layer_norm(y) * weight +
+    bias, in place, and the updated x is returned in ``out_dtype`` (x itself when that is fp32): the next sub-layer
+    reads the residual as it is.  Without ``y``: layer_norm(x) * weight + bias in ``out_dtype``; x stays.
+    Weight and bias are fp32 [W]."""
+    T, W = x.shape
+    if not _dev(x) or W * 4 > 60 * 1024:
+        return R.residual_layer_norm(x, y, weight, bias, eps, out_dtype)
+    assert x.dtype == torch.float32 and x.is_contiguous() and weight.dtype == torch.float32
+    assert bias is None or bias.dtype == torch.float32
+    h = None
+    if y is None or out_dtype != torch.float32:
+        h = torch.empty((T, W), dtype=out_dtype, device=x.device)
+    if y is not None:
+        assert y.stride(1) == 1 and y.shape == (T, W) and y.dtype == out_dtype
+    N.call("vda_residual_layer_norm", x.data_ptr(), N.ptr(y), y.stride(0) if y is not None else 0, weight.data_ptr(),
+           N.ptr(bias), N.ptr(h), W, float(eps), T, W, N.dt(out_dtype), N.stream())
+    return h if h is not None else x
+
+
+# ---- softmax attention with q / k norms, part-rotated heads, score maps, masks, sinks and an output gate ----------
+def qk_norm_rope_cache(qkv: torch.Tensor, H: int, G: int, D: int, Dv: int, maps: int, q_weight: torch.Tensor,
+                       k_weight: torch.Tensor, cos_sin: Optional[torch.Tensor], positions: torch.Tensor, rot: int,
+                       eps: float, k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+                       slot_mapping: torch.Tensor) -> torch.Tensor:
+    """qkv [T, >= H*maps*D + G*maps*D + G*Dv] (queries, keys, values side by side; further columns are ignored).  Every
+    D-wide map of every query / key head is divided by its root mean square, multiplied by q_weight / k_weight (fp32
+    [D]), and its first ``rot`` values are rotated in the half-split layout (value i pairs with i + rot / 2; cos_sin fp32
+    [positions, rot], cosines then sines).  Returns the queries [T, H, maps * D]; keys go to k_cache [blocks, G, bs,
+    maps * D] and values to v_cache [blocks, G, Dv, bs] at ``slot_mapping`` (negative: skipped)."""
+    used = (H + G) * maps * D + G * Dv
+    if not _dev(qkv):
+        return R.qk_norm_rope_cache(qkv[:, :used], H, G, D, Dv, maps, q_weight, k_weight, cos_sin, positions, rot, eps,
+                                    k_cache, v_cache, slot_mapping)
+    T = qkv.shape[0]
+    assert qkv.stride(1) == 1 and qkv.shape[1] >= used
+    assert k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype and slot_mapping.dtype == torch.int64
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and positions.dtype == torch.int64
+    bs = k_cache.shape[2]
+    assert k_cache.shape[1:] == (G, bs, maps * D) and v_cache.shape[1:] == (G, Dv, bs)
+    assert q_weight.dtype == torch.float32 and k_weight.dtype == torch.float32
+    assert rot == 0 or (cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and cos_sin.shape[1] == rot)
+    qn = torch.empty((T, H, maps * D), dtype=qkv.dtype, device=qkv.device)
+    N.call("vda_qk_norm_rope_cache", qn.data_ptr(), qkv.data_ptr(), qkv.stride(0), q_weight.data_ptr(),
+           k_weight.data_ptr(), N.ptr(cos_sin), positions.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+           slot_mapping.data_ptr(), T, H, G, D, Dv, maps, rot, bs, float(eps), N.dt(qkv.dtype), N.stream())
+    return qn
+
+
+def masked_softmax_attention(qn: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                             block_table: torch.Tensor, seq_lens: torch.Tensor, query_start_loc: torch.Tensor,
+                             scale: float, window: int = 0, chunk: int = 0, sink: Optional[torch.Tensor] = None,
+                             maps: int = 1, lam: Optional[torch.Tensor] = None, eps: float = 0.0,
+                             out_scale: float = 1.0, gate: Optional[torch.Tensor] = None, max_query_len: int = 1,
+                             out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """Causal softmax attention of qn [T, H, maps * D] over the paged keys and values (k_cache [blocks, G, bs, maps * D],
+    v_cache [blocks, G, Dv, bs]).  Key j is visible to the query at position i when j <= i, i - j < window (window > 0)
+    and j // chunk == i // chunk (chunk > 0).  ``sink`` fp32 [H]: exp(sink[h]) joins head h's denominator.  maps == 2:
+    two score maps per head over the same values, o = a1 - lam * a2 (``lam``: fp32 tensor of one element), then
+    o / rms(o) * out_scale over Dv.  ``gate`` [T, H * Dv] (row stride arbitrary): the result times sigmoid(gate).
+    Returns [T, H * Dv] in ``out_dtype`` (default: qn's type).  Scores, softmax and sums in fp32."""
+    out_dtype = out_dtype or qn.dtype
+    if not _dev(qn):
+        return R.masked_softmax_attention(qn, k_cache, v_cache, block_table, seq_lens, query_start_loc, scale, window,
+                                          chunk, sink, maps, lam, eps, out_scale, gate, out_dtype)
+    T, H, MD = qn.shape
+    G, Dv, bs = v_cache.shape[1], v_cache.shape[2], v_cache.shape[3]
+    assert qn.is_contiguous() and k_cache.is_contiguous() and v_cache.is_contiguous() and MD % maps == 0
+    assert qn.dtype == k_cache.dtype == v_cache.dtype == out_dtype and k_cache.shape[1:] == (G, bs, MD)
+    assert sink is None or (sink.dtype == torch.float32 and sink.numel() == H)
+    assert maps == 1 or (lam is not None and lam.dtype == torch.float32 and lam.is_cuda)
+    assert gate is None or (gate.dtype == qn.dtype and gate.stride(1) == 1 and gate.shape[1] == H * Dv)
+    out = torch.zeros((T, H * Dv), dtype=out_dtype, device=qn.device)
+    N.call("vda_masked_softmax_attention", out.data_ptr(), qn.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+           block_table.data_ptr(), block_table.stride(0), seq_lens.data_ptr(), query_start_loc.data_ptr(),
+           N.ptr(sink), N.ptr(lam), N.ptr(gate), gate.stride(0) if gate is not None else 0, float(scale), int(window),
+           int(chunk), int(maps), float(eps), float(out_scale), seq_lens.shape[0], H, G, MD // maps, Dv, bs,
+           max(int(max_query_len), 1), N.dt(out_dtype), N.stream())
     return out

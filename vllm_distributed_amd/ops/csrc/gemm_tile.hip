@@ -41,7 +41,9 @@
 // moe_align_block_size (csrc/moe/moe_align_sum_kernels.cu:17-230).
 #include "mfma_tile.h"
 
-enum { EPI_PLAIN = 0, EPI_GATE_UP = 1, EPI_DOWN = 2 };
+// EPI_UP_ACT: the first GEMM of experts without a gate half (rows gathered per pair like EPI_GATE_UP, plain weight
+// rows, act(v) out)
+enum { EPI_PLAIN = 0, EPI_GATE_UP = 1, EPI_DOWN = 2, EPI_UP_ACT = 3 };
 enum { SC_NONE = 0, SC_TOKEN = 1, SC_BLOCK = 2 };
 
 struct TileGemmArgs {
@@ -130,7 +132,7 @@ __global__ __launch_bounds__(512, 1) void tile_gemm_kernel(const TileGemmArgs a)
     long row = pos;
     if (GROUPED) {
       const int p = a.sorted[pos];
-      row = EPI == EPI_GATE_UP ? p / a.top_k : p;
+      row = (EPI == EPI_GATE_UP || EPI == EPI_UP_ACT) ? p / a.top_k : p;
     }
     xsrc[j] = xbase + row * a.x_stride * EB + ((slot ^ swz(tau)) << 4);
   }
@@ -178,7 +180,7 @@ __global__ __launch_bounds__(512, 1) void tile_gemm_kernel(const TileGemmArgs a)
       long row = pos;
       if (GROUPED) {
         const int p = a.sorted[pos];
-        row = EPI == EPI_GATE_UP ? p / a.top_k : p;
+        row = (EPI == EPI_GATE_UP || EPI == EPI_UP_ACT) ? p / a.top_k : p;
       }
       xs_row[nt] = a.x_scale + row * kblocks;
     }
@@ -249,7 +251,7 @@ __global__ __launch_bounds__(512, 1) void tile_gemm_kernel(const TileGemmArgs a)
     if (GROUPED) {
       const int p = a.sorted[beg + tau];
       orow = p;
-      if (SC == SC_TOKEN) s *= a.x_scale[EPI == EPI_GATE_UP ? p / a.top_k : p];
+      if (SC == SC_TOKEN) s *= a.x_scale[(EPI == EPI_GATE_UP || EPI == EPI_UP_ACT) ? p / a.top_k : p];
       if (EPI == EPI_DOWN) tw = a.topk_w[p];
     } else if (SC == SC_TOKEN) {
       s *= a.x_scale[orow];
@@ -280,6 +282,7 @@ __global__ __launch_bounds__(512, 1) void tile_gemm_kernel(const TileGemmArgs a)
         for (int i = 0; i < 4; ++i) {
           float v = acc[mt][nt][i] * s * tw;
           if (EPI == EPI_PLAIN && a.bias) v += n + 3 < a.N ? (float)bv[i] : (n + i < a.N ? (float)reinterpret_cast<const TO*>(a.bias)[n + i] : 0.f);
+          if (EPI == EPI_UP_ACT) v = gate_act(v, a.act);
           o[i] = (TO)v;
         }
         if (n + 3 < a.N) *reinterpret_cast<V4*>(op + n) = o;
@@ -411,6 +414,7 @@ static int launch_tile_gemm(const TileGemmArgs& a, int epi, bool grouped, int ro
   if (grouped) {
     if (epi == EPI_GATE_UP) BY_TN(EPI_GATE_UP, true);
     else if (epi == EPI_DOWN) BY_TN(EPI_DOWN, true);
+    else if (epi == EPI_UP_ACT) BY_TN(EPI_UP_ACT, true);
     else return -4;
   } else {
     if (epi != EPI_PLAIN) return -4;

@@ -1,0 +1,349 @@
+// Softmax attention on the paged cache with the pieces several decoder designs combine freely:
+//   * per-head RMS norms of queries and keys with a learned weight, then a rotation of the first `rot` values of a
+//     head in the half-split layout (value i pairs with value i + rot / 2), angles from an fp32 cos | sin table;
+//   * key and value widths of their own (D, Dv), grouped query heads;
+//   * `maps` score maps per head over the same values (maps = 2: differential attention, o = a1 - lam * a2, divided
+//     by its root mean square over Dv and scaled);
+//   * masks: causal, and on top a sliding window (i - j < window) and / or chunks counted from the sequence's start
+//     (j / chunk == i / chunk);
+//   * a sink per head: exp(sink[h]) joins the softmax denominator, with no key and no value;
+//   * an output gate: the result times the sigmoid of a second projection.
+//
+// Cache layout: k_cache [blocks, G, bs, maps * D] (a head's maps side by side in one row), v_cache [blocks, G, Dv, bs].
+//
+//   vda_qk_norm_rope_cache         per token: norms, rotation, the query rows out, key rows and values into the cache
+//   vda_masked_softmax_attention   plain fp32 arithmetic for any sizes and types: one workgroup per (sequence, tile of
+//                                  query tokens, group of heads that share a key / value head) walks the visible keys
+//                                  in tiles through LDS with a running maximum and sum per row; keys outside the mask
+//                                  of the tile's first query are never loaded.  Prompts, portions and single decoded
+//                                  tokens are one code path; keys are added in a fixed order per (token, head, map),
+//                                  so a result does not depend on how a prompt was cut or batched.
+#include "common.h"
+
+template <typename T>
+__global__ __launch_bounds__(256) void qk_norm_rope_cache_kernel(
+    T* __restrict__ qn, const T* __restrict__ qkv, long qkv_stride, const float* __restrict__ q_w,
+    const float* __restrict__ k_w, const float* __restrict__ cos_sin, const long* __restrict__ positions,
+    T* __restrict__ k_cache, T* __restrict__ v_cache, const long* __restrict__ slot_mapping, int H, int G, int D,
+    int Dv, int maps, int rot, int bs, float eps) {
+  const long t = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const T* row = qkv + t * qkv_stride;
+  const int half = rot / 2;
+  const float* cs = rot > 0 ? cos_sin + positions[t] * (long)rot : nullptr;
+  const long slot = slot_mapping[t];
+  const int nq = H * maps, nk = G * maps;
+  // one wave per D-wide unit: the query maps first, then the key maps
+  for (int u = wave; u < nq + nk; u += 4) {
+    const bool is_q = u < nq;
+    const T* src = row + (long)u * D;             // q units and k units are contiguous in the row
+    const float* w = is_q ? q_w : k_w;
+    float ss = 0.f;
+    for (int d = lane; d < D; d += 64) {
+      const float v = (float)src[d];
+      ss += v * v;
+    }
+    ss = wave_sum(ss);
+    const float rs = 1.f / sqrtf(ss / (float)D + eps);
+    T* dst;
+    if (is_q) {
+      dst = qn + (t * nq + u) * (long)D;
+    } else {
+      if (slot < 0) continue;
+      const int uk = u - nq;                      // key unit = head * maps + map
+      const int g = uk / maps, mp = uk % maps;
+      dst = k_cache + (((slot / bs) * G + g) * (long)bs + slot % bs) * (long)(maps * D) + (long)mp * D;
+    }
+    for (int d = lane; d < D; d += 64) {
+      float v = (float)src[d] * rs * w[d];
+      if (d < rot) {
+        const int i = d < half ? d : d - half;
+        const int pd = d < half ? d + half : d - half;
+        const float o = (float)src[pd] * rs * w[pd];
+        const float co = cs[i], si = cs[half + i];
+        v = d < half ? v * co - o * si : v * co + o * si;
+      }
+      dst[d] = (T)v;
+    }
+  }
+  if (slot >= 0) {
+    const T* vsrc = row + (long)(nq + nk) * D;
+    T* vdst = v_cache + (slot / bs) * (long)G * Dv * bs + slot % bs;      // [blocks, G, Dv, bs]
+    for (int e = tid; e < G * Dv; e += 256) vdst[(long)e * bs] = vsrc[e];
+  }
+}
+
+VDA_EXPORT int vda_qk_norm_rope_cache(void* qn, const void* qkv, long qkv_stride, const float* q_w, const float* k_w,
+                                      const float* cos_sin, const long* positions, void* k_cache, void* v_cache,
+                                      const long* slot_mapping, int T, int H, int G, int D, int Dv, int maps, int rot,
+                                      int bs, float eps, int dtype, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (rot < 0 || rot > D || (rot & 1) || maps < 1 || (rot > 0 && !cos_sin)) return -1;
+#define L(TT) hipLaunchKernelGGL((qk_norm_rope_cache_kernel<TT>), dim3(T), dim3(256), 0, st, (TT*)qn, (const TT*)qkv,  \
+                                 qkv_stride, q_w, k_w, cos_sin, positions, (TT*)k_cache, (TT*)v_cache, slot_mapping,  \
+                                 H, G, D, Dv, maps, rot, bs, eps)
+  if (dtype == VDA_BF16) L(bf16_t);
+  else if (dtype == VDA_F16) L(f16_t);
+  else if (dtype == VDA_F32) L(float);
+  else return -3;
+#undef L
+  VDA_CHECK_LAUNCH();
+  return 0;
+}
+
+struct MaskedAttnArgs {
+  void* out;                 // [T, H * Dv]
+  const void* qn;            // [T, H, maps * D]
+  const void* k_cache;
+  const void* v_cache;
+  const int* block_table;
+  long bt_stride;
+  const int* seq_lens;
+  const int* qsl;
+  const float* sink;         // [H] or null
+  const float* lam;          // one value (maps == 2)
+  const void* gate;          // [T, H * Dv] pre-activations or null
+  long gate_stride;
+  float scale, eps, out_scale;
+  int window, chunk, maps;
+  int H, G, D, Dv, bs;
+  int HG;                    // heads per workgroup (of the H / G that share a key / value head)
+  int BQ, BK;
+};
+
+// first key position the query at position p can see
+__device__ __forceinline__ int mask_lower(int p, int window, int chunk) {
+  int lo = 0;
+  if (window > 0) lo = max(lo, p - window + 1);
+  if (chunk > 0) lo = max(lo, p / chunk * chunk);
+  return lo;
+}
+
+// NACC: output values per thread (M * Dv <= 256 * NACC); M = BQ * heads * maps rows per workgroup (at most 256)
+template <typename T, int NACC>
+__global__ __launch_bounds__(256) void masked_softmax_attention_kernel(const MaskedAttnArgs a) {
+  const int R = a.H / a.G;                      // query heads per key / value head
+  const int ngr = (R + a.HG - 1) / a.HG;
+  const int g = blockIdx.z / ngr;
+  const int hl0 = (blockIdx.z % ngr) * a.HG;    // first of this workgroup's heads inside the group
+  const int HN = min(a.HG, R - hl0);
+  const int maps = a.maps, D = a.D, Dv = a.Dv, bs = a.bs, BQ = a.BQ, BK = a.BK;
+  const int MD = maps * D;
+  extern __shared__ float lds[];
+  const int Dq = D | 1;                         // odd row pitch: no bank conflicts when lanes walk rows
+  const int Kq = MD | 1, Vq = Dv | 1, RS = BK + 1;
+  const int M = BQ * HN * maps;                 // row m = (i * HN + hl) * maps + map
+  float* qs = lds;                              // [M][Dq]
+  float* ks = qs + BQ * a.HG * maps * Dq;       // [BK][Kq]
+  float* vs = ks + BK * Kq;                     // [BK][Vq]
+  float* sc = vs + BK * Vq;                     // [M][RS] scores, then weights
+  float* rm = sc + BQ * a.HG * maps * RS;       // [M] running maximum
+  float* rl = rm + BQ * a.HG * maps;            // [M] running sum
+  float* ra = rl + BQ * a.HG * maps;            // [M] rescale of this tile
+
+  const int s = blockIdx.y, tid = threadIdx.x;
+  const int sl = a.seq_lens[s];
+  if (sl <= 0) return;
+  const int t0 = a.qsl[s], L = a.qsl[s + 1] - t0;
+  const int i0 = blockIdx.x * BQ;
+  if (i0 >= L) return;
+  const int nq = min(BQ, L - i0);
+  const int p0 = sl - L + i0, p1 = p0 + nq;      // positions of the tile's queries: [p0, p1)
+  const int* bt = a.block_table + (long)s * a.bt_stride;
+  const T* qn = (const T*)a.qn;
+  const T* kc = (const T*)a.k_cache;
+  const T* vc = (const T*)a.v_cache;
+  const int h0 = g * R + hl0;
+
+  for (int e = tid; e < M * D; e += 256) {
+    const int d = e % D, m = e / D;
+    const int mp = m % maps, hl = (m / maps) % HN, i = m / (maps * HN);
+    qs[m * Dq + d] = i < nq ? (float)qn[((long)(t0 + i0 + i) * a.H + h0 + hl) * MD + mp * D + d] * a.scale : 0.f;
+  }
+  for (int m = tid; m < M; m += 256) {
+    const int hl = (m / maps) % HN;
+    if (a.sink) { rm[m] = a.sink[h0 + hl]; rl[m] = 1.f; }       // exp(sink - sink): the sink's share of the sum
+    else { rm[m] = -INFINITY; rl[m] = 0.f; }
+  }
+  float acc[NACC];
+#pragma unroll
+  for (int n = 0; n < NACC; ++n) acc[n] = 0.f;
+
+  const int lo = mask_lower(p0, a.window, a.chunk);
+  const int ntiles = (p1 - lo + BK - 1) / BK;
+  for (int tile = 0; tile < ntiles; ++tile) {
+    const int j0 = lo + tile * BK;
+    const int nk = min(BK, p1 - j0);
+    __syncthreads();
+    for (int e = tid; e < BK * MD; e += 256) {
+      const int d = e % MD, jj = e / MD;
+      float v = 0.f;
+      if (jj < nk) {
+        const int j = j0 + jj;
+        v = (float)kc[(((long)bt[j / bs] * a.G + g) * bs + j % bs) * MD + d];
+      }
+      ks[jj * Kq + d] = v;
+    }
+    for (int e = tid; e < BK * Dv; e += 256) {
+      const int jj = e % BK, d = e / BK;          // consecutive threads walk the keys of one value channel
+      float v = 0.f;
+      if (jj < nk) {
+        const int j = j0 + jj;
+        v = (float)vc[(((long)bt[j / bs] * a.G + g) * Dv + d) * bs + j % bs];
+      }
+      vs[jj * Vq + d] = v;
+    }
+    __syncthreads();
+    for (int e = tid; e < M * BK; e += 256) {
+      const int jj = e % BK, m = e / BK;
+      const int i = m / (maps * HN);
+      const int pi = p0 + i, j = j0 + jj;
+      float sv = -INFINITY;
+      if (i < nq && jj < nk && j <= pi && j >= mask_lower(pi, a.window, a.chunk)) {
+        const float* qp = qs + m * Dq;
+        const float* kp = ks + jj * Kq + (m % maps) * D;
+        sv = 0.f;
+        for (int d = 0; d < D; ++d) sv += qp[d] * kp[d];
+      }
+      sc[m * RS + jj] = sv;
+    }
+    __syncthreads();
+    // running maximum and sum per row; scores become weights relative to the new maximum
+    for (int m = tid; m < M; m += 256) {
+      float* sp = sc + m * RS;
+      float mx = rm[m];
+      for (int jj = 0; jj < nk; ++jj) mx = fmaxf(mx, sp[jj]);
+      const float mu = mx == -INFINITY ? 0.f : mx;
+      const float al = expf(rm[m] - mu);        // rm = -inf: 0
+      float sum = 0.f;
+      for (int jj = 0; jj < nk; ++jj) {
+        const float w = expf(sp[jj] - mu);
+        sp[jj] = w;
+        sum += w;
+      }
+      rm[m] = mx;
+      rl[m] = rl[m] * al + sum;
+      ra[m] = al;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int n = 0; n < NACC; ++n) {
+      const int e = tid + n * 256;
+      if (e < M * Dv) {
+        const int d = e % Dv, m = e / Dv;
+        const float* wp = sc + m * RS;
+        const float* vp = vs + d;
+        float v = acc[n] * ra[m];
+        for (int jj = 0; jj < nk; ++jj) v += wp[jj] * vp[jj * Vq];
+        acc[n] = v;
+      }
+    }
+  }
+  __syncthreads();
+  // normalised sums through LDS (over the tiles' space), then per (token, head): the maps' combination, its norm,
+  // the gate and the store; one wave per (token, head) at a time
+  float* oa = lds;                               // [M][Dv]
+#pragma unroll
+  for (int n = 0; n < NACC; ++n) {
+    const int e = tid + n * 256;
+    if (e < M * Dv) {
+      const float l = rl[e / Dv];
+      acc[n] = l > 0.f ? acc[n] / l : 0.f;
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int n = 0; n < NACC; ++n) {
+    const int e = tid + n * 256;
+    if (e < M * Dv) oa[e] = acc[n];
+  }
+  __syncthreads();
+  const int lane = tid & 63, wave = tid >> 6;
+  const float lam = maps == 2 ? *a.lam : 0.f;
+  T* out = (T*)a.out;
+  const T* gate = (const T*)a.gate;
+  for (int r = wave; r < nq * HN; r += 4) {
+    const int hl = r % HN, i = r / HN;
+    const float* a1 = oa + (long)(r * maps) * Dv;
+    const long tok = t0 + i0 + i;
+    const long col = (long)(h0 + hl) * Dv;
+    float rsn = 1.f;
+    if (maps == 2) {
+      float ss = 0.f;
+      for (int d = lane; d < Dv; d += 64) {
+        const float o = a1[d] - lam * a1[Dv + d];
+        ss += o * o;
+      }
+      ss = wave_sum(ss);
+      rsn = a.out_scale / sqrtf(ss / (float)Dv + a.eps);
+    }
+    for (int d = lane; d < Dv; d += 64) {
+      float o = maps == 2 ? (a1[d] - lam * a1[Dv + d]) * rsn : a1[d];
+      if (gate) o *= 1.f / (1.f + expf(-(float)gate[tok * a.gate_stride + col + d]));
+      out[tok * ((long)a.H * Dv) + col + d] = (T)o;
+    }
+  }
+}
+
+VDA_EXPORT int vda_masked_softmax_attention(void* out, const void* qn, const void* k_cache, const void* v_cache,
+                                            const int* block_table, long bt_stride, const int* seq_lens,
+                                            const int* qsl, const float* sink, const float* lam, const void* gate,
+                                            long gate_stride, float scale, int window, int chunk, int maps, float eps,
+                                            float out_scale, int S, int H, int G, int D, int Dv, int bs, int max_q,
+                                            int dtype, hipStream_t st) {
+  if (S <= 0 || max_q <= 0) return 0;
+  if (H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0 || maps < 1 || maps > 2 || (maps == 2 && !lam)) return -1;
+  // tile sizes: the largest query tile (then key tile) whose accumulators fit 64 registers per thread, whose rows
+  // fit one workgroup and whose tiles fit 96 KiB of LDS; single decoded tokens take a one-token tile; the heads of
+  // a group are dealt to several workgroups when one token's heads alone are too many for that
+  const int R = H / G, MD = maps * D;
+  const int Dq = D | 1, Kq = MD | 1, Vq = Dv | 1;
+  auto lds_of = [&](int bq, int bk, int hg) {
+    const size_t M = (size_t)bq * hg * maps;
+    const size_t main = M * Dq + (size_t)bk * Kq + (size_t)bk * Vq + M * (bk + 1) + 3 * M;
+    const size_t epi = M * Dv;
+    return (main > epi ? main : epi) * 4;
+  };
+  int BQ = 0, BK = 0, HG = R;
+  for (; HG >= 1 && !BQ; HG = HG > 1 ? (HG + 1) / 2 : 0) {
+    for (int bq = 16; bq >= 1 && !BQ; bq >>= 1) {
+      if (bq > 1 && bq / 2 >= max_q) continue;
+      const size_t M = (size_t)bq * HG * maps;
+      if (M * Dv > 256 * 64 || M > 256) continue;
+      for (int bk = 64; bk >= 8; bk >>= 1)
+        if (lds_of(bq, bk, HG) <= 96 * 1024) { BQ = bq; BK = bk; break; }
+    }
+    if (BQ) break;
+  }
+  if (!BQ) return -2;
+  const size_t lds = lds_of(BQ, BK, HG);
+  const int per = (BQ * HG * maps * Dv + 255) / 256;
+  const int NACC = per <= 8 ? 8 : per <= 16 ? 16 : per <= 32 ? 32 : 64;
+  MaskedAttnArgs a;
+  a.out = out; a.qn = qn; a.k_cache = k_cache; a.v_cache = v_cache; a.block_table = block_table;
+  a.bt_stride = bt_stride; a.seq_lens = seq_lens; a.qsl = qsl; a.sink = sink; a.lam = lam; a.gate = gate;
+  a.gate_stride = gate_stride; a.scale = scale; a.eps = eps; a.out_scale = out_scale; a.window = window;
+  a.chunk = chunk; a.maps = maps; a.H = H; a.G = G; a.D = D; a.Dv = Dv; a.bs = bs; a.HG = HG; a.BQ = BQ; a.BK = BK;
+  dim3 grid((max_q + BQ - 1) / BQ, S, G * ((R + HG - 1) / HG)), block(256);
+#define L2(TT, NA)                                                                                                  \
+  do {                                                                                                              \
+    if (lds > 48 * 1024) {                                                                                          \
+      hipError_t e = hipFuncSetAttribute((const void*)masked_softmax_attention_kernel<TT, NA>,                      \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                     \
+      if (e != hipSuccess) return (int)e;                                                                           \
+    }                                                                                                               \
+    hipLaunchKernelGGL((masked_softmax_attention_kernel<TT, NA>), grid, block, lds, st, a);                         \
+  } while (0)
+#define L(TT)                                                                                                       \
+  do {                                                                                                              \
+    if (NACC == 8) L2(TT, 8); else if (NACC == 16) L2(TT, 16); else if (NACC == 32) L2(TT, 32); else L2(TT, 64);    \
+  } while (0)
+  if (dtype == VDA_BF16) L(bf16_t);
+  else if (dtype == VDA_F16) L(f16_t);
+  else if (dtype == VDA_F32) L(float);
+  else return -3;
+#undef L
+#undef L2
+  VDA_CHECK_LAUNCH();
+  return 0;
+}

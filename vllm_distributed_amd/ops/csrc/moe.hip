@@ -550,11 +550,13 @@ VDA_EXPORT int vda_moe_sum(void* out, const void* out2, const int* ids, int num_
 // pair walks its expert's rows with plain dot products, a wave per row, lanes along K.  No sorting, no host
 // synchronisation, so it is also what a captured decode step launches for such experts.
 //   vda_moe_pairs: part[p, :] = topk_w[p] * W2_e (pair(Wg_e x_t, Wu_e x_t)),  out[t] = sum over the token's pairs
+//   (gated = 0: experts without a gate half, W2_e act(Wu_e x_t), w13 then holds I rows per expert)
 template <typename T>
 __global__ __launch_bounds__(256) void moe_pair_kernel(float* __restrict__ part, const T* __restrict__ x, long x_stride,
                                                        const T* __restrict__ w13, const T* __restrict__ w2,
                                                        const float* __restrict__ topk_w, const int* __restrict__ ids,
-                                                       int H, int I, int Ho, int k, int act_kind, float act_limit) {
+                                                       int H, int I, int Ho, int k, int act_kind, float act_limit,
+                                                       int gated) {
   extern __shared__ float lds[];
   float* xs = lds;              // [H]
   float* mid = lds + H;         // [I]
@@ -569,18 +571,22 @@ __global__ __launch_bounds__(256) void moe_pair_kernel(float* __restrict__ part,
   const T* xr = x + (p / k) * x_stride;
   for (int c = tid; c < H; c += 256) xs[c] = (float)xr[c];
   __syncthreads();
-  const T* wg = w13 + (long)e * 2 * I * H;
+  const T* wg = w13 + (long)e * (gated ? 2 : 1) * I * H;
   for (int j = wave; j < I; j += 4) {
     const T* g = wg + (long)j * H;
-    const T* u = wg + (long)(I + j) * H;
     float a = 0.f, b = 0.f;
-    for (int c = lane; c < H; c += 64) {
-      a += (float)g[c] * xs[c];
-      b += (float)u[c] * xs[c];
+    if (gated) {
+      const T* u = wg + (long)(I + j) * H;
+      for (int c = lane; c < H; c += 64) {
+        a += (float)g[c] * xs[c];
+        b += (float)u[c] * xs[c];
+      }
+      b = wave_sum(b);
+    } else {
+      for (int c = lane; c < H; c += 64) a += (float)g[c] * xs[c];
     }
     a = wave_sum(a);
-    b = wave_sum(b);
-    if (lane == 0) mid[j] = gated_pair(a, b, act_kind, act_limit);
+    if (lane == 0) mid[j] = gated ? gated_pair(a, b, act_kind, act_limit) : gate_act(a, act_kind);
   }
   __syncthreads();
   const T* wd = w2 + (long)e * Ho * I;
@@ -607,14 +613,15 @@ __global__ __launch_bounds__(256) void moe_pair_sum_kernel(T* __restrict__ out, 
 
 VDA_EXPORT int vda_moe_pairs(void* out, long out_stride, float* part, const void* x, long x_stride, const void* w13,
                              const void* w2, const float* topk_w, const int* ids, int T, int H, int I, int Ho, int k,
-                             int act_kind, float act_limit, int dtype, hipStream_t st) {
+                             int act_kind, float act_limit, int gated, int dtype, hipStream_t st) {
   if (T <= 0) return 0;
   const size_t lds = (size_t)(H + I) * 4;
   if (lds > 60 * 1024 || k < 1) return -1;
 #define L(TT)                                                                                                         \
   do {                                                                                                                \
     hipLaunchKernelGGL((moe_pair_kernel<TT>), dim3((unsigned)((long)T * k)), dim3(256), lds, st, part, (const TT*)x,   \
-                       x_stride, (const TT*)w13, (const TT*)w2, topk_w, ids, H, I, Ho, k, act_kind, act_limit);       \
+                       x_stride, (const TT*)w13, (const TT*)w2, topk_w, ids, H, I, Ho, k, act_kind, act_limit,        \
+                       gated);                                                                                        \
     hipLaunchKernelGGL((moe_pair_sum_kernel<TT>), dim3(T), dim3(256), 0, st, (TT*)out, out_stride, part, Ho, k);      \
   } while (0)
   if (dtype == VDA_BF16) L(bf16_t);

@@ -313,3 +313,70 @@ VDA_EXPORT int vda_residual_norms(float* x, const void* y, long y_stride, const 
   VDA_CHECK_LAUNCH();
   return 0;
 }
+
+// fp32 residual whose sub-layers are normed on their OUTPUT: x += (y - mean(y)) / sqrt(var(y) + eps) * w + b, in place,
+// and the updated row goes out once more in the activation type, as the next sub-layer's input (one launch for the
+// norm, the residual sum and the cast).  Without y: h = layer norm of x itself (the model's last norm), x stays.
+// The source row sits in LDS between the passes (mean, squared deviations, output).
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void residual_layer_norm_kernel(float* __restrict__ x, const T* __restrict__ y,
+                                                                  long y_stride, const float* __restrict__ w,
+                                                                  const float* __restrict__ b, T* __restrict__ h,
+                                                                  long h_stride, float eps, int W) {
+  extern __shared__ float row[];
+  __shared__ float red[16];
+  const long t = blockIdx.x;
+  const int tid = threadIdx.x;
+  float* xr = x + t * W;
+  const T* yr = y ? y + t * y_stride : nullptr;
+  float s = 0.f;
+  for (int c = tid * VEC; c < W; c += 256 * VEC) {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      const float v = yr ? (float)yr[c + i] : xr[c + i];
+      row[c + i] = v;
+      s += v;
+    }
+  }
+  const float mean = block_sum(s, red) / (float)W;
+  float ss = 0.f;
+  for (int c = tid * VEC; c < W; c += 256 * VEC) {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      const float d = row[c + i] - mean;
+      ss += d * d;
+    }
+  }
+  const float r = 1.f / sqrtf(block_sum(ss, red) / (float)W + eps);
+  for (int c = tid * VEC; c < W; c += 256 * VEC) {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      float v = (row[c + i] - mean) * r * w[c + i] + (b ? b[c + i] : 0.f);
+      if (yr) {
+        v += xr[c + i];
+        xr[c + i] = v;
+      }
+      if (h) h[t * h_stride + c + i] = (T)v;
+    }
+  }
+}
+
+VDA_EXPORT int vda_residual_layer_norm(float* x, const void* y, long y_stride, const float* w, const float* b,
+                                       void* h, long h_stride, float eps, int T, int W, int dtype, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (!w || (!y && !h)) return -1;
+  const size_t lds = (size_t)W * 4;
+  if (lds > 60 * 1024) return -2;
+  const bool vec = W % 4 == 0 && y_stride % 4 == 0 && h_stride % 4 == 0;
+#define L2(TT, VV) hipLaunchKernelGGL((residual_layer_norm_kernel<TT, VV>), dim3(T), dim3(256), lds, st, x,          \
+                                      (const TT*)y, y_stride, w, b, (TT*)h, h_stride, eps, W)
+#define L(TT) do { if (vec) L2(TT, 4); else L2(TT, 1); } while (0)
+  if (dtype == VDA_BF16) L(bf16_t);
+  else if (dtype == VDA_F16) L(f16_t);
+  else if (dtype == VDA_F32) L(float);
+  else return -3;
+#undef L
+#undef L2
+  VDA_CHECK_LAUNCH();
+  return 0;
+}

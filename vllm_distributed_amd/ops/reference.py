@@ -377,13 +377,15 @@ def moe_topk_softmax(logits: torch.Tensor, k: int, renormalize: bool):
 
 def fused_moe(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, topk_w: torch.Tensor, topk_ids: torch.Tensor,
               w13_scale: Optional[torch.Tensor] = None, w2_scale: Optional[torch.Tensor] = None,
-              block_scales: bool = False, activation: str = "silu", act_limit: float = 0.0) -> torch.Tensor:
+              block_scales: bool = False, activation: str = "silu", act_limit: float = 0.0,
+              gated: bool = True) -> torch.Tensor:
     """out[t] = sum_j topk_w[t, j] * W2_e( act(Wg_e x_t) * (Wu_e x_t) ), e = topk_ids[t, j];
     negative ids (expert on another rank) contribute nothing.  fp32 accumulation.  ``block_scales``:
-    the weight scales are per 128 x 128 block instead of per expert."""
+    the weight scales are per 128 x 128 block instead of per expert.  ``gated=False``: experts without a gate half,
+    W2_e act(Wu_e x_t), w13 [E, I, H]."""
     T, H = x.shape
     E, I2, _ = w13.shape
-    I = I2 // 2
+    I = I2 // 2 if gated else I2
     out = torch.zeros((T, w2.shape[1]), dtype=torch.float32, device=x.device)
     xf = x.float()
     for e in range(E):
@@ -401,7 +403,9 @@ def fused_moe(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, topk_w: torc
             q, s_ = per_group_fp8_quant(xe.to(x.dtype))
             xe = (q.float().view(*s_.shape, -1) * s_.unsqueeze(-1)).view(xe.shape)
         h = xe @ a.t()
-        if activation == "clamped_swiglu":
+        if not gated:
+            act = _act(activation, h).to(x.dtype).float()
+        elif activation == "clamped_swiglu":
             act = clamped_swiglu(h[:, :I], h[:, I:], act_limit).to(x.dtype).float()
         else:
             act = (_act(activation, h[:, :I]) * h[:, I:]).to(x.dtype).float()
@@ -799,3 +803,111 @@ def mlstm(proj, i_bias, f_bias, norm_w, state_nm, state_s, qsl, seq_lens, slot_t
     o = out * torch.rsqrt(out.pow(2).mean(-1, keepdim=True) + eps)
     o = o.view(T, HV) * norm_w.float() * torch.sigmoid(og)
     return o.to(proj.dtype)
+
+
+# ---- fp32 residual with a layer norm on every sub-layer's output -------------------------------------------------
+def residual_layer_norm(x, y, weight, bias, eps: float, out_dtype):
+    """x fp32 [T, W].  With ``y`` (a sub-layer's output): x += (y - mean) / sqrt(var + eps) * weight + bias, in place, and
+    x comes back in ``out_dtype`` (the next sub-layer reads the residual itself).  Without: the layer norm of x comes
+    back in ``out_dtype`` and x stays."""
+    src = y.float() if y is not None else x
+    mu = src.mean(-1, keepdim=True)
+    d = src - mu
+    n = d * torch.rsqrt(d.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
+    if bias is not None:
+        n = n + bias.float()
+    if y is None:
+        return n.to(out_dtype)
+    x += n
+    return x if out_dtype == torch.float32 else x.to(out_dtype)
+
+
+# ---- softmax attention with per-head q / k norms, part-rotated heads, several score maps and a choice of masks ---
+def rotate_halves(x, cos, sin, rot: int):
+    """x [..., D]: value i < rot / 2 is paired with value i + rot / 2 and the pair turned by the angle whose cos / sin
+    [..., rot / 2] are given (fp32); values from ``rot`` on pass unchanged."""
+    half = rot // 2
+    u, v = x[..., :half].float(), x[..., half:rot].float()
+    return torch.cat((u * cos - v * sin, v * cos + u * sin, x[..., rot:].float()), dim=-1)
+
+
+def qk_norm_rope_cache(qkv, H: int, G: int, D: int, Dv: int, maps: int, q_weight, k_weight, cos_sin, positions,
+                       rot: int, eps: float, k_cache, v_cache, slot_mapping):
+    """qkv [T, H*maps*D + G*maps*D + G*Dv].  Every D-wide map of every query / key head is divided by its root mean
+    square, multiplied by q_weight / k_weight [D] and its first ``rot`` values are rotated (cos_sin fp32 [positions, rot],
+    cosines then sines).  Returns q [T, H, maps * D]; keys go to k_cache [blocks, G, bs, maps * D] and values to v_cache
+    [blocks, G, Dv, bs] at ``slot_mapping``."""
+    T = qkv.shape[0]
+    nq, nk = H * maps * D, G * maps * D
+    q = qkv[:, :nq].float().view(T, H * maps, D)
+    k = qkv[:, nq: nq + nk].float().view(T, G * maps, D)
+    v = qkv[:, nq + nk:].view(T, G, Dv)
+    q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * q_weight.float()
+    k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * k_weight.float()
+    if rot > 0:
+        cs = cos_sin[positions[:T].long()]
+        cos, sin = cs[:, None, : rot // 2], cs[:, None, rot // 2: rot]
+        q, k = rotate_halves(q, cos, sin, rot), rotate_halves(k, cos, sin, rot)
+    qn = q.to(qkv.dtype).view(T, H, maps * D)
+    if k_cache is not None:
+        bs = k_cache.shape[2]
+        ok = slot_mapping[:T] >= 0
+        slots = slot_mapping[:T][ok].long()
+        k_cache[slots // bs, :, slots % bs] = k.to(k_cache.dtype).view(T, G, maps * D)[ok]
+        v_cache[slots // bs, :, :, slots % bs] = v.to(v_cache.dtype)[ok]
+    return qn
+
+
+def masked_softmax_attention(qn, k_cache, v_cache, block_table, seq_lens, qsl, scale: float, window: int, chunk: int,
+                             sink, maps: int, lam, eps: float, out_scale: float, gate, out_dtype):
+    """Softmax attention of qn [T, H, maps * D] over the paged keys (k_cache [blocks, G, bs, maps * D], v_cache [blocks,
+    G, Dv, bs]); head h reads key / value head h // (H / G).  Key j is visible to the query at position i when j <= i,
+    i - j < window (window > 0) and j // chunk == i // chunk (chunk > 0).  ``sink`` fp32 [H]: exp(sink[h]) joins the
+    softmax denominator of head h (no key, no value).  maps == 2: each half of a head's row is an attention map of
+    its own over the same values, combined as o = a1 - lam * a2 (lam: fp32 tensor of one element), divided by its
+    root mean square over Dv and multiplied by out_scale.  ``gate`` [T, H * Dv]: the result is multiplied by its
+    sigmoid.  Returns [T, H * Dv] in ``out_dtype``."""
+    T, H, MD = qn.shape
+    D = MD // maps
+    G, Dv, bs = v_cache.shape[1], v_cache.shape[2], v_cache.shape[3]
+    rep = H // G
+    out = torch.zeros((T, H, Dv), dtype=torch.float32, device=qn.device)
+    for s in range(seq_lens.shape[0]):
+        sl = int(seq_lens[s])
+        t0, t1 = int(qsl[s]), int(qsl[s + 1])
+        L = t1 - t0
+        if sl <= 0 or L <= 0:
+            continue
+        nb = -(-sl // bs)
+        blocks = block_table[s, :nb].long()
+        keys = k_cache[blocks].permute(1, 0, 2, 3).reshape(G, nb * bs, MD)[:, :sl].float()
+        vals = v_cache[blocks].permute(1, 0, 3, 2).reshape(G, nb * bs, Dv)[:, :sl].float()
+        i = torch.arange(sl - L, sl, device=qn.device)[:, None]
+        j = torch.arange(sl, device=qn.device)[None, :]
+        vis = j <= i
+        if window > 0:
+            vis = vis & (i - j < window)
+        if chunk > 0:
+            vis = vis & (i // chunk == j // chunk)
+        q = qn[t0:t1].float().view(L, G, rep, maps, D)
+        sc = torch.einsum("igrmd,gjmd->grmij", q, keys.view(G, sl, maps, D)) * scale
+        sc = sc.masked_fill(~vis, float("-inf"))
+        mx = sc.max(-1, keepdim=True).values
+        if sink is not None:
+            sk = sink.float().view(G, rep, 1, 1, 1)
+            mx = torch.maximum(mx, sk)
+        e = torch.exp(sc - mx)
+        den = e.sum(-1, keepdim=True)
+        if sink is not None:
+            den = den + torch.exp(sk - mx)
+        a = torch.einsum("grmij,gjd->igrmd", e / den, vals)                  # [L, G, rep, maps, Dv]
+        if maps == 2:
+            o = a[..., 0, :] - lam.float().reshape(()) * a[..., 1, :]
+            o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * out_scale
+        else:
+            o = a[..., 0, :]
+        out[t0:t1] = o.reshape(L, H, Dv)
+    out = out.view(T, H * Dv)
+    if gate is not None:
+        out = out * torch.sigmoid(gate[:T].float())
+    return out.to(out_dtype)
