@@ -141,5 +141,6 @@ VDA_EXPORT int vda_activation(void* out, const void* in, long n, int act_kind, f
   if (n == 0) return 0;
   if (dtype == VDA_BF16) return launch_plain<bf16_t>(out, in, n, act_kind, threshold, st);
   if (dtype == VDA_F16) return launch_plain<f16_t>(out, in, n, act_kind, threshold, st);
+  if (dtype == VDA_F32) return launch_plain<float>(out, in, n, act_kind, threshold, st);
   return -3;
 }
