@@ -108,7 +108,7 @@ class MaskedSoftmaxAttention(nn.Module):
             self.lq1, self.lk1 = _fp32_param((D,), 0.0), _fp32_param((D,), 0.0)
             self.lq2, self.lk2 = _fp32_param((D,), 0.0), _fp32_param((D,), 0.0)
         self._lam: Optional[torch.Tensor] = None
-        if self.taps > 1:
+        if self.taps >= 1:
             dtype = torch.get_default_dtype()
             self.conv_weight = nn.Parameter(torch.zeros((self.qkv_width, self.taps), dtype=dtype), requires_grad=False)
             offs = [0, nq, nq + nk]
@@ -120,8 +120,9 @@ class MaskedSoftmaxAttention(nn.Module):
                     t = t.reshape(t.shape[0], -1)
                     param.data[offs[shard_id]: offs[shard_id] + t.shape[0]].copy_(t)
             set_weight_attrs(self.conv_weight, {"weight_loader": load_conv})
+            # one tap: a weight per channel, no earlier rows, nothing carried
             self.conv_states = nn.ModuleList([ShortConvState(self.qkv_width, self.taps, f"{prefix}.conv.{i}")
-                                              for i in range(users)])
+                                              for i in range(users if self.taps > 1 else 0)])
         self.caches = nn.ModuleList([PagedKV(G, maps * D, Dv, f"{prefix}.kv.{i}") for i in range(users)])
         self.max_len = int(get_current_vllm_config().model_config.max_model_len) + 1
         self._cos_sin: Optional[torch.Tensor] = None
@@ -162,6 +163,8 @@ class MaskedSoftmaxAttention(nn.Module):
             tbl = StateSpaceLayer.slot_table(md)[:S]
             qkv = ops.causal_conv1d(p[:n, :W], self.conv_weight, None, st.conv_state, qsl, lens, tbl,
                                     md.max_query_len, activation=False)
+        elif self.taps == 1:
+            qkv = (p[:n, :W].float() * self.conv_weight.float().view(1, -1)).to(p.dtype)
         qn = ops.qk_norm_rope_cache(qkv, H, G, D, Dv, maps, self.q_norm, self.k_norm, self._table(p.device),
                                     positions[:n], self.rot_dims, self.eps, kv.k_cache, kv.v_cache,
                                     md.slot_mapping[:n])

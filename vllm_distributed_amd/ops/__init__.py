@@ -1249,7 +1249,7 @@ def causal_conv1d(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Te
     conv_state [slots, C, W-1] holds the last W-1 inputs of every request and is rolled forward in place;
     sequence s uses slot ``block_table[s, 0]``, and rows with ``seq_lens[s] == 0`` are skipped."""
     S = seq_lens.shape[0]
-    if not _dev(x):
+    if not _dev(x) or weight.shape[1] > 8:          # the kernel is built for 2 ... 8 taps
         return R.causal_conv1d(x, weight, bias, conv_state, query_start_loc, seq_lens, block_table, activation)
     T, C = x.shape
     out = torch.empty((T, C), dtype=x.dtype, device=x.device)
