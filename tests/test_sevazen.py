@@ -36,6 +36,18 @@ def mixed_layers():
             O.window_layer(weights_of=1), O.diff_layer(weights_of=0), O.window_layer(weights_of=1)]
 
 
+def matrix_core_layers():
+    """Head widths the matrix-core attention kernels take in 16-bit runs (64 and 128 values for keys and values alike);
+    other runs take the kernel for any sizes."""
+    return [O.window_layer(heads=4, kv_heads=2, dim=64, vdim=64, window=21, rot_dims=32, mlp="dense"),
+            O.diff_layer(heads=2, kv_heads=1, dim=64, vdim=64, chunk=16, rot_dims=16, mlp="moe"),
+            O.diff_layer(heads=4, kv_heads=4, dim=128, vdim=128, chunk=40, rot_dims=128, mlp=None),
+            O.window_layer(heads=4, kv_heads=2, dim=64, vdim=64, window=21, rot_dims=32, mlp="dense", weights_of=0)]
+
+
+LAYER_SETS = {"mixed": mixed_layers, "matrix_core": matrix_core_layers}
+
+
 # ---- driving the engine ------------------------------------------------------------------------------------------
 def run_schedule(folder, dtype, device, prompts, schedule, max_tokens, block_size=16, eager=True):
     """``schedule``: steps of (request, token count); every request ends when its tokens are used up.  Returns
@@ -159,7 +171,9 @@ ATTN_SIZES = [(4, 2, 12, 20, 1, 9, 0, True, 8, False), (2, 1, 8, 12, 2, 0, 11, F
               (6, 2, 64, 64, 1, 40, 0, True, 32, False), (4, 2, 32, 64, 2, 0, 32, False, 8, True),
               (3, 3, 5, 7, 1, 0, 0, True, 0, False), (1, 1, 4, 2, 2, 1, 0, False, 4, False),
               (8, 1, 16, 16, 1, 33, 16, False, 16, True), (2, 2, 6, 70, 2, 0, 1, True, 2, False),
-              (16, 2, 128, 128, 2, 0, 64, False, 64, True)]
+              (16, 2, 128, 128, 2, 0, 64, False, 64, True), (4, 4, 64, 64, 2, 24, 16, False, 16, False),
+              (8, 2, 128, 128, 1, 30, 0, True, 128, True), (2, 1, 96, 96, 1, 0, 20, False, 0, False),
+              (12, 2, 64, 64, 1, 0, 0, True, 8, False)]
 
 
 @pytest.mark.parametrize("dev,dt", OP_CASES)
@@ -215,9 +229,11 @@ def test_masked_attention_paged(dev, dt, H, G, D, E, maps, window, chunk, sink, 
         from vllm_distributed_amd.layers.rotary import half_split_cos_sin
         cs = half_split_cos_sin(128, rot, 40.0, None, torch.device(dev))
 
+    mfma = ops.masked_attention_mfma_ok(H, G, D, E, maps, sink, dt, dev == "cuda")
+
     def write(r, pos, slots):
         return ops.qk_norm_rope_cache(r.to(dev), H, G, D, E, maps, qw.to(dev), kw.to(dev), cs, pos.to(dev), rot, eps,
-                                      kc, vc, slots.to(dev))
+                                      kc, vc, slots.to(dev), by_map=mfma)
     for s, (n, k) in enumerate(zip(lens, news)):          # context first, as earlier steps would have
         if n - k:
             pos = torch.arange(n - k)
@@ -230,8 +246,18 @@ def test_masked_attention_paged(dev, dt, H, G, D, E, maps, window, chunk, sink, 
     sl = torch.tensor(lens, dtype=torch.int32).to(dev)
     gt = torch.cat([g[n - k:] for g, n, k in zip(gates, lens, news)]).to(dev) if gate else None
     lam = torch.tensor([lam_v], device=dev) if maps == 2 else None
-    got = ops.masked_softmax_attention(qn, kc, vc, table.to(dev), sl, qsl, scale, window, chunk,
-                                       sk.to(dev) if sink else None, maps, lam, eps, out_scale, gt, max(news), dt)
+    if mfma:
+        # the matrix-core kernels: the decoded token through the decode form (whole, and with its keys dealt to three
+        # workgroups), the portion and the prompt through the tiled form
+        got = [ops.masked_softmax_attention_mfma(qn, kc, vc, table.to(dev), sl, qsl, qsl[1:] - 1, 1, 1, 2, sum(news[1:]),
+                                                 1, splits, max(news), scale, H, window, chunk,
+                                                 sk.to(dev) if sink else None, maps, lam, eps, out_scale, gt)
+               for splits in (1, 3)]
+        assert rel(got[1], got[0]) < 1e-2
+        got = got[0]
+    else:
+        got = ops.masked_softmax_attention(qn, kc, vc, table.to(dev), sl, qsl, scale, window, chunk,
+                                           sk.to(dev) if sink else None, maps, lam, eps, out_scale, gt, max(news), dt)
     assert rel(got, want) < OP_TOL[dt] * (3 if dt == torch.bfloat16 else 1)
 
 
@@ -341,6 +367,7 @@ VARIANTS = {
     "experts_plain": dict(layers=[O.diff_layer(mlp=O.feed_forward("moe", experts=5, top=1, shared=None)),
                                   O.window_layer(mlp=O.feed_forward("moe", experts=4, top=4, shared=8))],
                           width=40, vocab=50),
+    "matrix_core_sizes": dict(layers=matrix_core_layers()),
     "shared_weights_in_a_chain": dict(layers=[O.diff_layer(mlp="moe"), O.diff_layer(mlp="moe", weights_of=0),
                                               O.diff_layer(mlp="moe", weights_of=1)]),
 }
@@ -380,8 +407,9 @@ def test_residual_after_every_layer(tmp_path):
 
 
 @pytest.mark.parametrize("dev,dtype", CASES)
-def test_prefill_equals_decoding_token_by_token(tmp_path, dev, dtype):
-    folder, cfg, W = model(tmp_path, mixed_layers(), seed=4)
+@pytest.mark.parametrize("layers", list(LAYER_SETS))
+def test_prefill_equals_decoding_token_by_token(tmp_path, dev, dtype, layers):
+    folder, cfg, W = model(tmp_path, LAYER_SETS[layers](), seed=4)
     p = tokens(70, cfg["vocab"], 5)
     sched = [[("a", 11)]] + [[("a", 1)]] * 59          # decodes 59 tokens: six windows of 9, five chunks of 11
     got = run_schedule(folder, dtype, dev, {"a": p}, sched, 80)
@@ -393,8 +421,9 @@ def test_prefill_equals_decoding_token_by_token(tmp_path, dev, dtype):
 
 @pytest.mark.parametrize("dev,dtype", CASES)
 @pytest.mark.parametrize("block_size", [16, 32])
-def test_portions_down_to_two_tokens(tmp_path, dev, dtype, block_size):
-    folder, cfg, W = model(tmp_path, mixed_layers(), seed=6)
+@pytest.mark.parametrize("layers", list(LAYER_SETS))
+def test_portions_down_to_two_tokens(tmp_path, dev, dtype, block_size, layers):
+    folder, cfg, W = model(tmp_path, LAYER_SETS[layers](), seed=6)
     p = tokens(90, cfg["vocab"], 7)
     cuts = [2, 3, 11, 2, 16, 1, 17, 2, 7, 12, 1, 1, 15]
     assert sum(cuts) == 90
@@ -403,10 +432,11 @@ def test_portions_down_to_two_tokens(tmp_path, dev, dtype, block_size):
 
 
 @pytest.mark.parametrize("dev,dtype", CASES)
-def test_unequal_requests_share_steps_and_reuse_pages_and_slots(tmp_path, dev, dtype):
+@pytest.mark.parametrize("layers", list(LAYER_SETS))
+def test_unequal_requests_share_steps_and_reuse_pages_and_slots(tmp_path, dev, dtype, layers):
     """Seven requests over four slots and a pool of 10 pages: portions beside single tokens, requests that sit out
     steps, pages and slots of finished requests taken by later ones."""
-    folder, cfg, W = model(tmp_path, mixed_layers(), seed=8)
+    folder, cfg, W = model(tmp_path, LAYER_SETS[layers](), seed=8)
     V = cfg["vocab"]
     prompts = {"a": tokens(40, V, 1), "b": tokens(17, V, 2), "c": tokens(1, V, 3), "d": tokens(33, V, 4),
                "e": tokens(48, V, 5), "f": tokens(9, V, 6), "g": tokens(30, V, 7)}
@@ -502,10 +532,11 @@ def test_long_decoding(tmp_path):
 
 
 @pytest.mark.gpu
-def test_decode_graphs_equal_eager(tmp_path):
+@pytest.mark.parametrize("layers", list(LAYER_SETS))
+def test_decode_graphs_equal_eager(tmp_path, layers):
     """Single decoded tokens through captured graphs (several replays with other work between them) give the
     eager logits."""
-    folder, cfg, W = model(tmp_path, mixed_layers(), seed=10)
+    folder, cfg, W = model(tmp_path, LAYER_SETS[layers](), seed=10)
     V = cfg["vocab"]
     prompts = {"a": tokens(30, V, 1), "b": tokens(22, V, 2)}
     sched = [[("a", 10), ("b", 4)]] + [[("a", 1), ("b", 1)]] * 18 + [[("a", 2)]]

@@ -82,6 +82,7 @@ _REGISTRY: dict[str, tuple[Callable[[str], Any], Any]] = {
     "VDA_DENSE_GEMM_MAX_M": (int, 192),          # rows up to which 16-bit linears run the in-tree ping-pong MFMA GEMM (0 = never;
                                                  # at 256 rows the library's selected algorithms win inside the engine)
     "VDA_SIGMOID_ATTN_FORM": (str, "auto"),      # sigmoid head-mixing attention: auto | mfma | plain (fp32 arithmetic)
+    "VDA_MASKED_ATTN_FORM": (str, "auto"),       # softmax attention with sinks / chunks / score maps: auto | plain
     "VDA_DENSE_GEMM_MIN_M": (int, 33),           # below: the library GEMM is as fast or faster (measured, graph-captured layer chains)
     "VDA_DENSE_GEMM_MAX_N": (int, 16384),        # wider weight matrices (gate/up) fill the chip without a K split: library
     "VDA_DENSE_GATE_UP_MAX_M": (int, 0),         # rows up to which a gated MLP runs SiLU * up inside the GEMM epilogue (0 = never:

@@ -124,7 +124,13 @@ class MaskedSoftmaxAttention(nn.Module):
             self.conv_states = nn.ModuleList([ShortConvState(self.qkv_width, self.taps, f"{prefix}.conv.{i}")
                                               for i in range(users if self.taps > 1 else 0)])
         self.caches = nn.ModuleList([PagedKV(G, maps * D, Dv, f"{prefix}.kv.{i}") for i in range(users)])
-        self.max_len = int(get_current_vllm_config().model_config.max_model_len) + 1
+        cfg = get_current_vllm_config()
+        # 16-bit activations and head widths the matrix-core paged attention kernels are built for: those kernels (every
+        # score map a key head of its own in the cache); anything else, fp32 included: the kernel for any sizes
+        self.use_mfma = ops.masked_attention_mfma_ok(H, G, D, Dv, maps, bool(sink), cfg.model_config.dtype,
+                                                     cfg.device_config.device != "cpu") \
+            and cfg.cache_config.cache_dtype == "auto"
+        self.max_len = int(cfg.model_config.max_model_len) + 1
         self._cos_sin: Optional[torch.Tensor] = None
 
     def _table(self, device) -> Optional[torch.Tensor]:
@@ -165,6 +171,24 @@ class MaskedSoftmaxAttention(nn.Module):
                                     md.max_query_len, activation=False)
         elif self.taps == 1:
             qkv = (p[:n, :W].float() * self.conv_weight.float().view(1, -1)).to(p.dtype)
+        g_rows = gate[:n] if gate is not None else None
+        if self.use_mfma:
+            qn = ops.qk_norm_rope_cache(qkv, H, G, D, Dv, maps, self.q_norm, self.k_norm, self._table(p.device),
+                                        positions[:n], self.rot_dims, self.eps, kv.k_cache, kv.v_cache,
+                                        md.slot_mapping[:n], by_map=True)
+            nd, ndt, n_pre, npt, pqsl = (md.num_decode_seqs, md.num_decode_tokens, md.num_prefill_seqs,
+                                         md.num_prefill_tokens, md.prefill_query_start_loc)
+            cols = max(md.max_decode_query_len, 1) * (H // G)
+            if nd > 0 and (cols > 32 or (cols > 16 and D > 128)):
+                # more query rows per key head than the decode form takes: the tiled form serves every sequence
+                nd, ndt, n_pre, npt, pqsl = 0, 0, S, n, qsl
+            out = ops.masked_softmax_attention_mfma(
+                qn, kv.k_cache, kv.v_cache, md.block_table, md.seq_lens, md.query_start_loc, pqsl, nd, ndt, n_pre, npt,
+                md.max_decode_query_len, md.decode_num_splits, md.max_query_len, self.scale, H, self.window,
+                self.chunk, self.sink, maps, self._lambda(), self.eps, 1.0 - self.diff, g_rows)
+            if n < T:
+                out = torch.cat([out, out.new_zeros((T - n, out.shape[1]))], dim=0)
+            return self.o_proj(out)
         qn = ops.qk_norm_rope_cache(qkv, H, G, D, Dv, maps, self.q_norm, self.k_norm, self._table(p.device),
                                     positions[:n], self.rot_dims, self.eps, kv.k_cache, kv.v_cache,
                                     md.slot_mapping[:n])

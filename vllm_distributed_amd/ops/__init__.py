@@ -244,10 +244,15 @@ def decode_num_splits(num_seqs: int, num_kv_heads: int, max_seq_len: int) -> int
 def paged_attention_decode(out, q, k_cache, v_cache, block_table, seq_lens, q_start_loc, scale: float,
                            num_splits: int = 1, max_q_len: int = 1, window: int = 0, softcap: float = 0.0,
                            alibi: Optional[torch.Tensor] = None, workspace=None, k_scale: float = 1.0,
-                           v_scale: float = 1.0):
-    """q, out: [T, Hq, D].  Each sequence has <= max_q_len query tokens (1 for plain decode)."""
+                           v_scale: float = 1.0, sink: Optional[torch.Tensor] = None, chunk: int = 0,
+                           v_shift: int = 0):
+    """q, out: [T, Hq, D].  Each sequence has <= max_q_len query tokens (1 for plain decode).
+    ``sink`` fp32 [Hq]: exp(sink[h]) joins head h's softmax denominator; ``chunk`` > 0: keys of the query's own chunk
+    of that many positions only; ``v_shift``: K head k reads V head k >> v_shift (v_cache holds that many fewer heads).
+    These three are options of the device kernels only."""
     T, Hq, D = q.shape
     if not _dev(q):
+        assert sink is None and not chunk and not v_shift
         out.copy_(R.paged_attention(q, k_cache, v_cache, block_table, seq_lens, q_start_loc, scale, window,
                                     softcap, alibi, k_scale=k_scale, v_scale=v_scale))
         return out
@@ -263,14 +268,15 @@ def paged_attention_decode(out, q, k_cache, v_cache, block_table, seq_lens, q_st
            block_table.data_ptr(), seq_lens.data_ptr(), q_start_loc.data_ptr(), N.ptr(alibi), N.ptr(part_out),
            N.ptr(part_lse), S, T, Hq, k_cache.shape[1], D, k_cache.shape[2], block_table.stride(0), num_splits,
            max_q_len, q.stride(0), out.stride(0), scale, softcap, window, N.dt(q.dtype), _kv_fp8(k_cache), k_scale,
-           v_scale, N.stream())
+           v_scale, N.ptr(sink), int(chunk), int(v_shift), N.stream())
     return out
 
 
 def paged_attention_prefill(out, q, k_cache, v_cache, block_table, seq_lens, q_start_loc, scale: float,
                             window: int = 0, softcap: float = 0.0, alibi: Optional[torch.Tensor] = None,
                             k_scale: float = 1.0, v_scale: float = 1.0, causal: bool = True,
-                            return_lse: bool = False, max_q_len: int = 0):
+                            return_lse: bool = False, max_q_len: int = 0, sink: Optional[torch.Tensor] = None,
+                            chunk: int = 0, v_shift: int = 0):
     """Varlen attention of new tokens against the paged cache.  ``causal=False``: every query token sees
     all ``seq_lens[s]`` keys of its sequence (encoder models, the shared-prefix pass of cascade
     attention).  ``return_lse``: also return the log-sum-exp [Hq, T] (natural log) of every row.
@@ -278,6 +284,7 @@ def paged_attention_prefill(out, q, k_cache, v_cache, block_table, seq_lens, q_s
     the wide kernel then starts the longest causal tiles of all sequences first."""
     T, Hq, D = q.shape
     if not _dev(q):
+        assert sink is None and not chunk and not v_shift        # options of the device kernels (see the decode form)
         o, lse = R.paged_attention(q, k_cache, v_cache, block_table, seq_lens, q_start_loc, scale, window,
                                    softcap, alibi, return_lse=True, k_scale=k_scale, v_scale=v_scale,
                                    causal=causal)
@@ -288,7 +295,7 @@ def paged_attention_prefill(out, q, k_cache, v_cache, block_table, seq_lens, q_s
            block_table.data_ptr(), seq_lens.data_ptr(), q_start_loc.data_ptr(), N.ptr(alibi), seq_lens.shape[0], T,
            Hq, k_cache.shape[1], D, k_cache.shape[2], block_table.stride(0), q.stride(0), out.stride(0), scale,
            softcap, window, N.dt(q.dtype), _kv_fp8(k_cache), k_scale, v_scale, int(bool(causal)), N.ptr(lse),
-           int(max_q_len), N.stream())
+           int(max_q_len), N.ptr(sink), int(chunk), int(v_shift), N.stream())
     return (out, lse) if return_lse else out
 
 
@@ -1582,14 +1589,18 @@ def residual_layer_norm(x: torch.Tensor, y: Optional[torch.Tensor], weight: torc
 def qk_norm_rope_cache(qkv: torch.Tensor, H: int, G: int, D: int, Dv: int, maps: int, q_weight: torch.Tensor,
                        k_weight: torch.Tensor, cos_sin: Optional[torch.Tensor], positions: torch.Tensor, rot: int,
                        eps: float, k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
-                       slot_mapping: torch.Tensor) -> torch.Tensor:
+                       slot_mapping: torch.Tensor, by_map: bool = False) -> torch.Tensor:
     """qkv [T, >= H*maps*D + G*maps*D + G*Dv] (queries, keys, values side by side; further columns are ignored).  Every
     D-wide map of every query / key head is divided by its root mean square, multiplied by q_weight / k_weight (fp32
     [D]), and its first ``rot`` values are rotated in the half-split layout (value i pairs with i + rot / 2; cos_sin fp32
     [positions, rot], cosines then sines).  Returns the queries [T, H, maps * D]; keys go to k_cache [blocks, G, bs,
-    maps * D] and values to v_cache [blocks, G, Dv, bs] at ``slot_mapping`` (negative: skipped)."""
+    maps * D] and values to v_cache [blocks, G, Dv, bs] at ``slot_mapping`` (negative: skipped).
+    ``by_map`` (device kernels, for the matrix-core attention path): every map is a key head of its own, the same
+    k_cache memory read as [blocks, G * maps, bs, D], and the queries come back ordered (key head, map, head inside the
+    group) as [T, H * maps, D]."""
     used = (H + G) * maps * D + G * Dv
     if not _dev(qkv):
+        assert not by_map
         return R.qk_norm_rope_cache(qkv[:, :used], H, G, D, Dv, maps, q_weight, k_weight, cos_sin, positions, rot, eps,
                                     k_cache, v_cache, slot_mapping)
     T = qkv.shape[0]
@@ -1600,11 +1611,69 @@ def qk_norm_rope_cache(qkv: torch.Tensor, H: int, G: int, D: int, Dv: int, maps:
     assert k_cache.shape[1:] == (G, bs, maps * D) and v_cache.shape[1:] == (G, Dv, bs)
     assert q_weight.dtype == torch.float32 and k_weight.dtype == torch.float32
     assert rot == 0 or (cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and cos_sin.shape[1] == rot)
-    qn = torch.empty((T, H, maps * D), dtype=qkv.dtype, device=qkv.device)
+    qn = torch.empty((T, H * maps, D) if by_map else (T, H, maps * D), dtype=qkv.dtype, device=qkv.device)
     N.call("vda_qk_norm_rope_cache", qn.data_ptr(), qkv.data_ptr(), qkv.stride(0), q_weight.data_ptr(),
            k_weight.data_ptr(), N.ptr(cos_sin), positions.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
-           slot_mapping.data_ptr(), T, H, G, D, Dv, maps, rot, bs, float(eps), N.dt(qkv.dtype), N.stream())
+           slot_mapping.data_ptr(), T, H, G, D, Dv, maps, rot, bs, float(eps), int(by_map), N.dt(qkv.dtype),
+           N.stream())
     return qn
+
+
+MASKED_ATTN_MFMA_SIZES = (64, 96, 128, 192, 256)
+
+
+def masked_attention_mfma_ok(H: int, G: int, D: int, Dv: int, maps: int, sink: bool, dtype: torch.dtype,
+                             on_device: bool) -> bool:
+    """Can the matrix-core paged attention kernels (ops/csrc/attention.hip) serve this layer?  16-bit activations and
+    cache, keys and values of one width that those kernels are built for."""
+    return (on_device and not envs.VDA_FORCE_TORCH_OPS and envs.VDA_MASKED_ATTN_FORM != "plain"
+            and dtype in (torch.bfloat16, torch.float16) and D == Dv and D in MASKED_ATTN_MFMA_SIZES
+            and H // G <= 128 and not (maps == 2 and sink))
+
+
+def masked_softmax_attention_mfma(qn: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                                  block_table: torch.Tensor, seq_lens: torch.Tensor, query_start_loc: torch.Tensor,
+                                  prefill_query_start_loc: Optional[torch.Tensor], num_decode_seqs: int,
+                                  num_decode_tokens: int, num_prefill_seqs: int, num_prefill_tokens: int,
+                                  max_decode_query_len: int, decode_num_splits: int, max_query_len: int, scale: float,
+                                  H: int, window: int = 0, chunk: int = 0, sink: Optional[torch.Tensor] = None,
+                                  maps: int = 1, lam: Optional[torch.Tensor] = None, eps: float = 0.0,
+                                  out_scale: float = 1.0, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``masked_softmax_attention`` on the matrix cores: the framework's paged attention kernels (decode form for the
+    leading decode sequences of the step, tiled form for the prompts) with the window, chunk and sink as their
+    options, every score map as a key head of its own that shares its group's values, and one epilogue launch for the
+    maps' combination, norm and gate.  qn [T, H * maps, D] and k_cache in the ``by_map`` layout of
+    ``qk_norm_rope_cache``; returns [T, H * Dv]."""
+    T, Hq, D = qn.shape
+    nb, G, Dv, bs = v_cache.shape
+    assert Hq == H * maps and D == Dv and qn.is_contiguous() and k_cache.is_contiguous() and v_cache.is_contiguous()
+    kview = k_cache.view(nb, G * maps, bs, D)
+    a = torch.empty((T, Hq, D), dtype=qn.dtype, device=qn.device)
+    nd, ndt, n_pre = int(num_decode_seqs), int(num_decode_tokens), int(num_prefill_seqs)
+    R_ = H // G
+    kw = dict(window=int(window), sink=sink, chunk=int(chunk), v_shift=maps - 1)
+    cols = max(int(max_decode_query_len), 1) * R_
+    if nd > 0 and (cols > 32 or (cols > 16 and D > 128)):
+        raise ValueError(f"{cols} query columns per key head and step are beyond the decode form")
+    if nd > 0:
+        paged_attention_decode(a[:ndt], qn[:ndt], kview, v_cache, block_table[:nd], seq_lens[:nd],
+                               query_start_loc[:nd + 1], scale, num_splits=int(decode_num_splits),
+                               max_q_len=int(max_decode_query_len), **kw)
+    if n_pre > 0:
+        e = ndt + int(num_prefill_tokens)
+        paged_attention_prefill(a[ndt:e], qn[ndt:e], kview, v_cache, block_table[nd:nd + n_pre],
+                                seq_lens[nd:nd + n_pre], prefill_query_start_loc, scale,
+                                max_q_len=int(max_query_len), **kw)
+        if e < T:
+            a[e:].zero_()
+    if maps == 1 and gate is None:
+        return a.view(T, H * Dv)
+    out = torch.empty((T, H * Dv), dtype=qn.dtype, device=qn.device)
+    assert gate is None or (gate.dtype == qn.dtype and gate.stride(1) == 1 and gate.shape == (T, H * Dv))
+    N.call("vda_map_combine", out.data_ptr(), a.data_ptr(), N.ptr(lam), N.ptr(gate),
+           gate.stride(0) if gate is not None else 0, T, H, G, Dv, int(maps), float(eps), float(out_scale),
+           N.dt(qn.dtype), N.stream())
+    return out
 
 
 def masked_softmax_attention(qn: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,

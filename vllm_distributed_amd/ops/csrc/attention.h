@@ -28,6 +28,10 @@ struct AttnParams {
   int num_tokens;           // T (row length of lse_out)
   float* lse_out;           // [Hq, T] natural-log log-sum-exp per (head, token), or nullptr (prefill form)
   int max_q_len;            // longest query run of the batch when the host knows it, else 0 (wide prefill form)
+  // options of the layers that are built from this kernel family (zero / null: off)
+  const float* sink;        // [Hq]: exp(sink[h]) joins head h's softmax denominator, with no key and no value
+  int chunk;                // > 0: the query at position i sees keys j with j / chunk == i / chunk only
+  int v_shift;              // K head k reads V head k >> v_shift (the V cache then holds Hkv >> v_shift heads)
 };
 
 // Key selection of the sparse prefill form: per (sequence, head) a list of single key positions ("vertical" lines of

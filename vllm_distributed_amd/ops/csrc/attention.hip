@@ -64,7 +64,7 @@ __global__ __launch_bounds__(256) void paged_attn_kernel(AttnParams p) {
   // column c of the workgroup -> (query token c / G, head c % G)
   int limit[NCT], lower[NCT];
   long col_off[NCT];           // element offset of (token, head) in q / out
-  float slope[NCT];
+  float slope[NCT], sink_m[NCT];
   V8 qf[NCT][KS];
   int wave_hi = 0, wave_lo = 0x7fffffff;
 #pragma unroll
@@ -76,8 +76,13 @@ __global__ __launch_bounds__(256) void paged_attn_kernel(AttnParams p) {
     const bool valid = qt < qt_end && (SPLIT ? c < COLS : true);
     limit[ct] = valid ? (p.causal ? ctx + qt + 1 : seq_len) : 0;
     lower[ct] = (valid && p.window > 0) ? max(0, limit[ct] - p.window) : 0;
+    if (valid && p.chunk > 0) lower[ct] = max(lower[ct], (limit[ct] - 1) / p.chunk * p.chunk);
     const int head = kvh * G + h;
     slope[ct] = (p.alibi && valid) ? p.alibi[head] : 0.f;
+    // a sink is a score without key or value: the running maximum starts there and the sum with its weight of one
+    // (once per column: in the lane group that holds the sum's first part, and in split mode in one wave of one part)
+    sink_m[ct] = (p.sink && valid && (!SPLIT || (wave == 0 && blockIdx.z == 0))) ? p.sink[head] * 1.4426950408889634f
+                                                                                  : -INFINITY;
     const T* qp = (const T*)p.q + (long)(qs + (valid ? qt : q0)) * p.q_stride + (long)head * D + g * DQ;
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
@@ -109,13 +114,14 @@ __global__ __launch_bounds__(256) void paged_attn_kernel(AttnParams p) {
   f32x4 acc[NCT][NT];
 #pragma unroll
   for (int ct = 0; ct < NCT; ++ct) {
-    m[ct] = -INFINITY; l[ct] = 0.f;
+    m[ct] = sink_m[ct]; l[ct] = (sink_m[ct] != -INFINITY && g == 0) ? 1.f : 0.f;
 #pragma unroll
     for (int n = 0; n < NT; ++n) acc[ct][n] = f32x4{0, 0, 0, 0};
   }
 
   const CT* kc = (const CT*)p.k_cache;
   const CT* vc = (const CT*)p.v_cache;
+  const int hkv_v = p.Hkv >> p.v_shift, kvh_v = kvh >> p.v_shift;      // the value head behind this key head
   // K row of this lane inside a step: tile u, row r  <->  key 8*(r>>2) + 4u + (r&3)
   const int krow0 = 8 * (r >> 2) + (r & 3);
 
@@ -135,7 +141,7 @@ __global__ __launch_bounds__(256) void paged_attn_kernel(AttnParams p) {
     const int tok = step * 32 + 8 * g;
     const int bi = max(min(tok / BS, nblk_valid - 1), 0);
     const long blk = bt[bi];
-    const CT* vp = vc + ((blk * p.Hkv + kvh) * (long)D + r) * BS + (tok % BS);
+    const CT* vp = vc + ((blk * hkv_v + kvh_v) * (long)D + r) * BS + (tok % BS);
 #pragma unroll
     for (int n = 0; n < NT; ++n) vf[n] = KVLoad<T, F8>::ld(vp + (long)n * 16 * BS);
   };
@@ -352,7 +358,7 @@ __global__ __launch_bounds__(256, PREFILL_WGS_PER_CU) void paged_prefill_lds_ker
 
   int limit[NCT], lower[NCT];
   long col_off[NCT];
-  float slope[NCT];
+  float slope[NCT], sink_m[NCT];
   V8 qf[NCT][KS];
   int wave_hi = 0, wave_lo = 0x7fffffff;
 #pragma unroll
@@ -363,8 +369,10 @@ __global__ __launch_bounds__(256, PREFILL_WGS_PER_CU) void paged_prefill_lds_ker
     const bool valid = qt < qt_end;
     limit[ct] = valid ? (p.causal ? ctx + qt + 1 : seq_len) : 0;
     lower[ct] = (valid && p.window > 0) ? max(0, limit[ct] - p.window) : 0;
+    if (valid && p.chunk > 0) lower[ct] = max(lower[ct], (limit[ct] - 1) / p.chunk * p.chunk);
     const int head = head0 + h;
     slope[ct] = (p.alibi && valid) ? p.alibi[head] : 0.f;
+    sink_m[ct] = (p.sink && valid) ? p.sink[head] * 1.4426950408889634f : -INFINITY;
     const T* qp = (const T*)p.q + (long)(qs + (valid ? qt : q0)) * p.q_stride + (long)head * D + g * DQ;
 #pragma unroll
     for (int s = 0; s < KS; ++s) qf[ct][s] = valid ? ld16<V8>(qp + 8 * s) : V8{};
@@ -378,7 +386,8 @@ __global__ __launch_bounds__(256, PREFILL_WGS_PER_CU) void paged_prefill_lds_ker
   }
   // workgroup-uniform key range (all waves take part in every tile copy)
   const int wg_hi = p.causal ? ctx + qt_end : seq_len;
-  const int wg_lo = p.window > 0 ? max(0, ctx + q0 + 1 - p.window) : 0;
+  int wg_lo = p.window > 0 ? max(0, ctx + q0 + 1 - p.window) : 0;
+  if (p.chunk > 0 && p.causal) wg_lo = max(wg_lo, (ctx + q0) / p.chunk * p.chunk);
   const int step_lo = wg_lo / 32, step_hi = (wg_hi + 31) / 32;
 
   __shared__ unsigned bm[SPARSE ? SPARSE_BM_WORDS : 1];
@@ -414,7 +423,7 @@ __global__ __launch_bounds__(256, PREFILL_WGS_PER_CU) void paged_prefill_lds_ker
   f32x4 acc[NCT][NT];
 #pragma unroll
   for (int ct = 0; ct < NCT; ++ct) {
-    m[ct] = -INFINITY; l[ct] = 0.f;
+    m[ct] = sink_m[ct]; l[ct] = (sink_m[ct] != -INFINITY && g == 0) ? 1.f : 0.f;
 #pragma unroll
     for (int n = 0; n < NT; ++n) acc[ct][n] = f32x4{0, 0, 0, 0};
   }
@@ -429,8 +438,9 @@ __global__ __launch_bounds__(256, PREFILL_WGS_PER_CU) void paged_prefill_lds_ker
 #endif
   // Address arithmetic kept in 32 bits except for the one block-number x block-stride product (a single
   // v_mad_u64_u32): offsets inside a block fit 32 bits by construction.
-  const unsigned blk_stride = (unsigned)p.Hkv * BS * D;          // elements per cache block (K and V alike)
-  const unsigned k_head = (unsigned)kvh * BS * D, v_head = (unsigned)kvh * D * BS;
+  const unsigned blk_stride = (unsigned)p.Hkv * BS * D;          // elements per K cache block
+  const unsigned v_blk_stride = (unsigned)(p.Hkv >> p.v_shift) * D * BS;     // per V cache block (fewer heads when shared)
+  const unsigned k_head = (unsigned)kvh * BS * D, v_head = (unsigned)(kvh >> p.v_shift) * D * BS;
   auto gload = [&](int step, V8 (&rk)[KPT], V8 (&rv)[VPT]) {
     const int tb = step * 32;
 #pragma unroll
@@ -449,7 +459,7 @@ __global__ __launch_bounds__(256, PREFILL_WGS_PER_CU) void paged_prefill_lds_ker
       const int tok = tb + 8 * c;
       const unsigned blk = (unsigned)bt[max(min(tok / BS, nblk_valid - 1), 0)];
       const unsigned off = v_head + (unsigned)d * BS + (tok % BS);
-      rv[i] = KVLoad<T, F8>::ld(vc + (size_t)blk * blk_stride + off);
+      rv[i] = KVLoad<T, F8>::ld(vc + (size_t)blk * v_blk_stride + off);
     }
   };
   // XOR swizzle of the 16-byte pieces of a K row.  ds_read_b128 serves lanes {0-3,12-15,20-27},
@@ -770,14 +780,16 @@ VDA_EXPORT int vda_paged_attention_decode(
     const int* seq_lens, const int* q_start_loc, const float* alibi, float* part_out, float* part_lse,
     int num_seqs, int num_tokens, int Hq, int Hkv, int D, int block_size, int max_blocks, int nsplit,
     int max_q_len, long q_stride, long out_stride, float scale, float softcap, int window, int dtype,
-    int kv_fp8, float k_scale, float v_scale, hipStream_t st) {
+    int kv_fp8, float k_scale, float v_scale, const float* sink, int chunk, int v_shift, hipStream_t st) {
   if (Hq % Hkv) return -1;
+  if (chunk < 0 || v_shift < 0 || (Hkv >> v_shift) << v_shift != Hkv) return -7;
   if (nsplit < 1 || nsplit > 64) return -6;      // the reduce kernel keeps one partition per lane
   const int cols = max_q_len * (Hq / Hkv);
   if (cols > 32 || (cols > 16 && D > 128)) return -4;
   AttnParams p{q, k_cache, v_cache, out, part_out, part_lse, block_table, seq_lens, q_start_loc, alibi,
                num_seqs, Hq, Hkv, max_blocks, nsplit, q_stride, out_stride, scale * (kv_fp8 ? k_scale : 1.f), softcap,
                kv_fp8 ? v_scale : 1.f, window, 0, 1, num_tokens, nullptr};
+  p.sink = sink; p.chunk = chunk; p.v_shift = v_shift;
   const int form = cols <= 16 ? 0 : 1;
   int rc = dtype == VDA_BF16 ? dispatch_d<bf16_t>(p, D, block_size, form, num_seqs, st, kv_fp8)
                              : dispatch_d<f16_t>(p, D, block_size, form, num_seqs, st, kv_fp8);
@@ -817,18 +829,21 @@ VDA_EXPORT int vda_paged_attention_prefill(
     const int* seq_lens, const int* q_start_loc, const float* alibi, int num_seqs, int num_tokens,
     int Hq, int Hkv, int D, int block_size, int max_blocks, long q_stride, long out_stride, float scale,
     float softcap, int window, int dtype, int kv_fp8, float k_scale, float v_scale, int causal, float* lse_out,
-    int max_q_len, hipStream_t st) {
+    int max_q_len, const float* sink, int chunk, int v_shift, hipStream_t st) {
   if (Hq % Hkv) return -1;
   const int G = Hq / Hkv;
   if (G > 128) return -4;
-  if (!causal && window > 0) return -5;
+  if (!causal && (window > 0 || chunk > 0)) return -5;
+  if (chunk < 0 || v_shift < 0 || (Hkv >> v_shift) << v_shift != Hkv) return -7;
+  const bool extras = sink != nullptr || chunk > 0 || v_shift > 0;     // served by the 4-wave form only
   const int q_tile = 128 / G;     // 4 waves x 32 columns
   AttnParams p{q, k_cache, v_cache, out, nullptr, nullptr, block_table, seq_lens, q_start_loc, alibi,
                num_seqs, Hq, Hkv, max_blocks, 1, q_stride, out_stride, scale * (kv_fp8 ? k_scale : 1.f), softcap,
                kv_fp8 ? v_scale : 1.f, window, q_tile, causal, num_tokens, lse_out, max_q_len};
+  p.sink = sink; p.chunk = chunk; p.v_shift = v_shift;
   // Wide form (8 waves, 256 columns, 64-key tiles): head size 128 and enough query tiles to occupy the
   // chip (one workgroup per CU); short chunks keep the 4-wave form, which cuts them into more workgroups.
-  if (D == 128 && 256 % G == 0 && (g_prefill_variant == 1 || g_prefill_variant == 3)) {
+  if (!extras && D == 128 && 256 % G == 0 && (g_prefill_variant == 1 || g_prefill_variant == 3)) {
     const int wide_tile = 256 / G;
     const long wgs = (long)(num_tokens / wide_tile) * Hkv;
     if (g_prefill_variant == 3 || wgs >= g_prefill_wide_min_wgs) {
@@ -837,7 +852,7 @@ VDA_EXPORT int vda_paged_attention_prefill(
     }
   }
   const int grid_x = num_tokens / q_tile + num_seqs;
-  const int form = g_prefill_variant == 0 ? 2 : 3;
+  const int form = (g_prefill_variant == 0 && !extras) ? 2 : 3;
   return dtype == VDA_BF16 ? dispatch_d<bf16_t>(p, D, block_size, form, grid_x, st, kv_fp8)
                            : dispatch_d<f16_t>(p, D, block_size, form, grid_x, st, kv_fp8);
 }

@@ -10,8 +10,12 @@
 //   * an output gate: the result times the sigmoid of a second projection.
 //
 // Cache layout: k_cache [blocks, G, bs, maps * D] (a head's maps side by side in one row), v_cache [blocks, G, Dv, bs].
+// For the matrix-core kernels of attention.hip every map is a key head of its own instead (`by_map`): k_cache
+// [blocks, G * maps, bs, D], queries ordered (key head, map, head inside the group), so that query row q reads key
+// head q / (H / G) and that key head k reads value head k / maps; vda_map_combine folds their output.
 //
 //   vda_qk_norm_rope_cache         per token: norms, rotation, the query rows out, key rows and values into the cache
+//   vda_map_combine                the epilogue of the matrix-core path: maps' combination, its norm, the gate
 //   vda_masked_softmax_attention   plain fp32 arithmetic for any sizes and types: one workgroup per (sequence, tile of
 //                                  query tokens, group of heads that share a key / value head) walks the visible keys
 //                                  in tiles through LDS with a running maximum and sum per row; keys outside the mask
@@ -25,7 +29,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_kernel(
     T* __restrict__ qn, const T* __restrict__ qkv, long qkv_stride, const float* __restrict__ q_w,
     const float* __restrict__ k_w, const float* __restrict__ cos_sin, const long* __restrict__ positions,
     T* __restrict__ k_cache, T* __restrict__ v_cache, const long* __restrict__ slot_mapping, int H, int G, int D,
-    int Dv, int maps, int rot, int bs, float eps) {
+    int Dv, int maps, int rot, int bs, float eps, int by_map) {
   const long t = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const T* row = qkv + t * qkv_stride;
@@ -47,12 +51,18 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_kernel(
     const float rs = 1.f / sqrtf(ss / (float)D + eps);
     T* dst;
     if (is_q) {
-      dst = qn + (t * nq + u) * (long)D;
+      int uo = u;                                 // query unit = head * maps + map
+      if (by_map) {                               // ... or (key head, map, head inside its group)
+        const int R = H / G, h = u / maps, mp = u % maps;
+        uo = ((h / R) * maps + mp) * R + h % R;
+      }
+      dst = qn + (t * nq + uo) * (long)D;
     } else {
       if (slot < 0) continue;
       const int uk = u - nq;                      // key unit = head * maps + map
       const int g = uk / maps, mp = uk % maps;
-      dst = k_cache + (((slot / bs) * G + g) * (long)bs + slot % bs) * (long)(maps * D) + (long)mp * D;
+      dst = by_map ? k_cache + (((slot / bs) * nk + uk) * (long)bs + slot % bs) * (long)D
+                   : k_cache + (((slot / bs) * G + g) * (long)bs + slot % bs) * (long)(maps * D) + (long)mp * D;
     }
     for (int d = lane; d < D; d += 64) {
       float v = (float)src[d] * rs * w[d];
@@ -76,12 +86,12 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_kernel(
 VDA_EXPORT int vda_qk_norm_rope_cache(void* qn, const void* qkv, long qkv_stride, const float* q_w, const float* k_w,
                                       const float* cos_sin, const long* positions, void* k_cache, void* v_cache,
                                       const long* slot_mapping, int T, int H, int G, int D, int Dv, int maps, int rot,
-                                      int bs, float eps, int dtype, hipStream_t st) {
+                                      int bs, float eps, int by_map, int dtype, hipStream_t st) {
   if (T <= 0) return 0;
   if (rot < 0 || rot > D || (rot & 1) || maps < 1 || (rot > 0 && !cos_sin)) return -1;
 #define L(TT) hipLaunchKernelGGL((qk_norm_rope_cache_kernel<TT>), dim3(T), dim3(256), 0, st, (TT*)qn, (const TT*)qkv,  \
                                  qkv_stride, q_w, k_w, cos_sin, positions, (TT*)k_cache, (TT*)v_cache, slot_mapping,  \
-                                 H, G, D, Dv, maps, rot, bs, eps)
+                                 H, G, D, Dv, maps, rot, bs, eps, by_map)
   if (dtype == VDA_BF16) L(bf16_t);
   else if (dtype == VDA_F16) L(f16_t);
   else if (dtype == VDA_F32) L(float);
@@ -344,6 +354,56 @@ VDA_EXPORT int vda_masked_softmax_attention(void* out, const void* qn, const voi
   else return -3;
 #undef L
 #undef L2
+  VDA_CHECK_LAUNCH();
+  return 0;
+}
+
+// a [T, G, maps, R, Dv] (the matrix-core kernels' output with one query row per map) -> out [T, H * Dv]:
+// o = a1 - lam * a2 divided by its root mean square over Dv and scaled (maps == 2), times sigmoid(gate).
+// One wave per (token, head).
+template <typename T>
+__global__ __launch_bounds__(256) void map_combine_kernel(T* __restrict__ out, const T* __restrict__ a,
+                                                          const float* __restrict__ lam_p, const T* __restrict__ gate,
+                                                          long gate_stride, long n_rows, int H, int G, int Dv,
+                                                          int maps, float eps, float out_scale) {
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= n_rows) return;
+  const int lane = threadIdx.x & 63;
+  const long t = row / H;
+  const int h = (int)(row % H), R = H / G;
+  const T* a1 = a + ((t * G + h / R) * maps * R + h % R) * (long)Dv;
+  const T* a2 = a1 + (long)R * Dv;
+  const float lam = maps == 2 ? *lam_p : 0.f;
+  float rsn = 1.f;
+  if (maps == 2) {
+    float ss = 0.f;
+    for (int d = lane; d < Dv; d += 64) {
+      const float o = (float)a1[d] - lam * (float)a2[d];
+      ss += o * o;
+    }
+    ss = wave_sum(ss);
+    rsn = out_scale / sqrtf(ss / (float)Dv + eps);
+  }
+  for (int d = lane; d < Dv; d += 64) {
+    float o = maps == 2 ? ((float)a1[d] - lam * (float)a2[d]) * rsn : (float)a1[d];
+    if (gate) o *= 1.f / (1.f + expf(-(float)gate[t * gate_stride + (long)h * Dv + d]));
+    out[row * Dv + d] = (T)o;
+  }
+}
+
+VDA_EXPORT int vda_map_combine(void* out, const void* a, const float* lam, const void* gate, long gate_stride, int T,
+                               int H, int G, int Dv, int maps, float eps, float out_scale, int dtype, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (H % G || maps < 1 || maps > 2 || (maps == 2 && !lam)) return -1;
+  const long rows = (long)T * H;
+#define L(TT) hipLaunchKernelGGL((map_combine_kernel<TT>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st,         \
+                                 (TT*)out, (const TT*)a, lam, (const TT*)gate, gate_stride, rows, H, G, Dv, maps, eps, \
+                                 out_scale)
+  if (dtype == VDA_BF16) L(bf16_t);
+  else if (dtype == VDA_F16) L(f16_t);
+  else if (dtype == VDA_F32) L(float);
+  else return -3;
+#undef L
   VDA_CHECK_LAUNCH();
   return 0;
 }

@@ -38,9 +38,10 @@ _SIGS = {
     "vda_transfer_blocks": [P, P, P, P, I, L, P],
     "vda_transfer_blocks_ex": [P, P, P, P, I, L, L, L, L, L, P],
     "vda_gather_cache": [P, P, P, P, P, I, I, I, I, I, P],
-    "vda_paged_attention_decode": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, L, L, F, F, I, I, I, F, F, P],
+    "vda_paged_attention_decode": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, L, L, F, F, I, I, I, F, F, P, I,
+                                   I, P],
     "vda_paged_attention_prefill": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, L, L, F, F, I, I, I, F, F, I, P,
-                                    I, P],
+                                    I, P, I, I, P],
     "vda_paged_attention_prefill_sparse": [P] * 13 + [I] * 9 + [L, L, F, F, I, I, F, F, I, P, L, P],
     "vda_set_prefill_variant": [I],
     "vda_int8_quant_azp": [P, P, P, P, P, P, I, I, L, L, I, P],
@@ -66,7 +67,8 @@ _SIGS = {
     "vda_group_rms_norm": [P, L, P, L, P, F, I, I, I, I, I, P],
     "vda_moe_pairs": [P, L, P, P, L, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
     "vda_residual_layer_norm": [P, P, L, P, P, P, L, F, I, I, I, P],
-    "vda_qk_norm_rope_cache": [P, P, L, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, I, P],
+    "vda_qk_norm_rope_cache": [P, P, L, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, I, I, P],
+    "vda_map_combine": [P, P, P, P, L, I, I, I, I, I, F, F, I, P],
     "vda_masked_softmax_attention": [P, P, P, P, P, L, P, P, P, P, P, L, F, I, I, I, F, F, I, I, I, I, I, I, I, I, P],
     "vda_moe_gate_up": [P, P, P, P, P, P, I, I, I, I, I, L, I, I, I, I, F, P],
     "vda_moe_down": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
