@@ -146,7 +146,10 @@ def main() -> None:
     ap.add_argument("--compare-rapovik", action="store_true",
                     help="likewise for Rapovik stacks (latent window attention, Mamba-2, mLSTM, routed experts) beside "
                          "a Jamba stack with routed experts of equal width, depth and feed-forward")
-    ap.add_argument("--sizes", default="small,medium", help="--compare-nositar / --compare-rapovik: small, medium, large")
+    ap.add_argument("--compare-sevazen", action="store_true",
+                    help="likewise for Sevazen stacks (window attention with sinks, differential attention in chunks, "
+                         "routed squared-ReLU experts) beside a sliding-window Mixtral stack of equal size")
+    ap.add_argument("--sizes", default="small,medium", help="--compare-...: small, medium, large")
     ap.add_argument("--rehearse-on-one-gpu", action="store_true", help="--disagg: every engine on GPU 0")
     ap.add_argument("--kv-push", action="store_true", help="--disagg: push blocks while prefilling (landing pool)")
     ap.add_argument("--num-prompts", type=int, default=200, help="--disagg: requests")
@@ -154,9 +157,10 @@ def main() -> None:
     a = ap.parse_args()
     if a.disagg:
         return run_disagg(a)
-    if a.compare_nositar or a.compare_rapovik:
+    if a.compare_nositar or a.compare_rapovik or a.compare_sevazen:
         from vllm_distributed_amd.benchmarks import hybrid_compare
-        argv = (["--models", "rapovik,jamba-moe"] if a.compare_rapovik else []) + ["--sizes", a.sizes, "--batch", str(32 if a.batch == 256 else a.batch),
+        argv = (["--models", "rapovik,jamba-moe"] if a.compare_rapovik else
+                ["--models", "sevazen,mixtral-swa"] if a.compare_sevazen else []) + ["--sizes", a.sizes, "--batch", str(32 if a.batch == 256 else a.batch),
                 "--input-len", str(2048 if a.input_len == 1024 else a.input_len),
                 "--output-len", str(64 if a.output_len == 128 else a.output_len)]
         hybrid_compare.main(argv + (["--enforce-eager"] if a.enforce_eager else []))

@@ -299,7 +299,7 @@ def make_weights(cfg, seed=0, dtype=torch.bfloat16):
             W[p + "mix.sink"] = vec(H, 0.5, 1.0)
         else:
             for n in ("lq1", "lk1", "lq2", "lk2"):
-                W[p + "mix." + n] = vec(D, 0.0, 0.3)
+                W[p + "mix." + n] = vec(D, 0.0, 0.5 / D ** 0.25)          # their dot products: about +- 0.25
             W[p + "mix.g"] = lin(H * E, Wd, 2.0)
         mlp = spec.get("mlp")
         if mlp is None:

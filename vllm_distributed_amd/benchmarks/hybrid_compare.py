@@ -1,8 +1,9 @@
-"""Prefill and decode throughput of a Nositar or Rapovik stack beside the closest existing models of equal size, random
+"""Prefill and decode throughput of a Nositar, Rapovik or Sevazen stack beside the closest existing models of equal size, random
 weights.
 
     python bench.py --compare-nositar [--sizes small,medium] [--batch 32] [--input-len 2048] [--output-len 64]
     python bench.py --compare-rapovik [...]        (rapovik beside jamba-moe)
+    python bench.py --compare-sevazen [...]        (sevazen beside mixtral-swa)
 
 Per size three engines run one after the other, each in a process of its own (``--one`` is the child's entry):
   nositar      alternating sigmoid head-mixing attention (window + kept first tokens) and gated delta-rule layers,
@@ -13,6 +14,11 @@ Per size three engines run one after the other, each in a process of its own (``
   jamba-moe    the same with 8 routed experts (two per token) in every other layer
   rapovik      latent window attention, Mamba-2 and mLSTM mixers in turn over an fp32 residual with norms around every
                sub-layer; clamped gated feed-forwards, dense and routed (8 experts, two per token, one shared) in turn
+  sevazen      window attention with sinks and a short convolution and differential attention inside chunks in turn,
+               fp32 residual with layer norms on the sub-layers' outputs, 8 routed squared-ReLU experts (two per token)
+               plus a shared expert in every layer
+  mixtral-swa  a Mixtral stack of the same width, depth and heads with the same sliding window and 8 routed gated
+               experts (two per token) of equal weight count
 Prefill: ``batch`` prompts of ``input-len`` tokens, one generated token.  Decode: the same requests generating
 ``output-len`` tokens, the prefill time taken off.  One JSON line per (size, model).
 """
@@ -92,7 +98,37 @@ def rapovik_config(s: dict) -> dict:
             "layers": [dict(cycle[i % 4], mlp=dense if i % 2 == 0 else moe) for i in range(s["layers"])]}
 
 
-MODELS = {"nositar": nositar_config, "llama-swa": llama_config, "jamba": jamba_config, "jamba-moe": jamba_moe_config,
+def mixtral_swa_config(s: dict) -> dict:
+    """A Mixtral stack with a sliding window: softmax attention + 8 routed gated experts (two per token) per layer."""
+    return {"architectures": ["MixtralForCausalLM"], "model_type": "mixtral", "hidden_size": s["width"],
+            "intermediate_size": s["ff"], "num_hidden_layers": s["layers"], "num_attention_heads": s["heads"],
+            "num_key_value_heads": s["kv_heads"], "head_dim": s["dim"], "vocab_size": s["vocab"],
+            "num_local_experts": 8, "num_experts_per_tok": 2, "sliding_window": s["window"],
+            "max_position_embeddings": 32768, "rms_norm_eps": 1e-6, "rope_theta": 10000.0,
+            "tie_word_embeddings": False, "torch_dtype": "bfloat16"}
+
+
+def sevazen_config(s: dict) -> dict:
+    """Window attention (sink, 4-tap convolution, half of each head rotated) and differential attention inside chunks of
+    the window's size (half as many heads: two score maps each) in turn; every layer has 8 routed squared-ReLU experts
+    (two per token; 1.5 x the width of the gated experts beside them, for equal weights) and a shared expert."""
+    w, ff, d = s["width"], s["ff"], s["dim"]
+    moe = {"kind": "moe", "router": {"experts": 8, "top": 2}, "expert": {"ff": ff * 3 // 2}, "shared": {"ff": ff // 4}}
+    win = {"type": "attention",
+           "mixer": {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": d, "vdim": d, "scale": d ** -0.5, "conv": 4,
+                     "mask": {"size": s["window"]},
+                     "rot": {"base": 500000.0, "dims": d // 2,
+                             "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}}
+    dif = {"type": "attention_2",
+           "mixer": {"heads": s["heads"] // 2, "kv_heads": max(s["kv_heads"] // 2, 1), "dim": d, "vdim": d,
+                     "scale": d ** -0.5, "diff": 0.5, "mask": {"size": s["window"]},
+                     "rot": {"base": 10000.0, "dims": d // 2,
+                             "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}}
+    return {"architecture": "Sevazen", "vocab": s["vocab"], "width": w, "norm": {"eps": 1e-6},
+            "layers": [dict(win if i % 2 == 0 else dif, mlp=moe) for i in range(s["layers"])]}
+
+
+MODELS = {"sevazen": sevazen_config, "mixtral-swa": mixtral_swa_config, "nositar": nositar_config, "llama-swa": llama_config, "jamba": jamba_config, "jamba-moe": jamba_moe_config,
           "rapovik": rapovik_config}
 
 
