@@ -132,6 +132,20 @@ def test_residual_with_output_layer_norm(dev, dt, W_):
     last = ops.residual_layer_norm(xd, None, w.to(dev), b.to(dev), eps, dt)   # the model's last norm: x stays
     torch.testing.assert_close(xd.cpu(), want, atol=2e-5, rtol=1e-5)
     assert rel(last, O.layer_norm(want, w, b, eps)) < OP_TOL[dt]
+    # a second part of the sub-layer's output behind a one-number-per-row sigmoid gate, formed in the same pass
+    y2, gate = torch.randn(T, W_).to(dt), torch.randn(T, 3)
+    want2 = x + O.layer_norm(y.float() + y2.float() * torch.sigmoid(gate[:, 2:]), w, b, eps)
+    xd = x.clone().to(dev)
+    ops.residual_layer_norm(xd, y.to(dev), w.to(dev), b.to(dev), eps, dt, y2.to(dev), gate.to(dev)[:, 2:])
+    torch.testing.assert_close(xd.cpu(), want2, atol=2e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("dev,dt", OP_CASES)
+def test_fp32_dot_products_of_16_bit_rows(dev, dt):
+    x, w, b = torch.randn(9, 77).to(dt), torch.randn(5, 77), torch.randn(5)
+    got = ops.fp32_rows_dot(x.to(dev)[:, :70], w[:, :70].contiguous().to(dev), b.to(dev))
+    assert got.dtype == torch.float32
+    torch.testing.assert_close(got.cpu(), x[:, :70].float() @ w[:, :70].T + b, atol=1e-4, rtol=1e-5)
 
 
 def rot_table(rot, kind, n, dev):

@@ -30,13 +30,12 @@ from typing import Iterable, Optional
 
 import torch
 import torch.nn as nn
-import torch.nn.functional as F
 
 from .. import ops
 from ..config import VllmConfig
 from ..layers.basic import LogitsProcessor, ParallelLMHead, VocabParallelEmbedding
 from ..layers.hyper_connections import _fp32_param
-from ..layers.linear import ColumnParallelLinear, ReplicatedLinear, RowParallelLinear, default_weight_loader
+from ..layers.linear import ColumnParallelLinear, RowParallelLinear, default_weight_loader, set_weight_attrs
 from ..layers.masked_attention import MaskedSoftmaxAttention
 from ..layers.moe import FusedMoE
 
@@ -128,22 +127,31 @@ class SevazenMoE(nn.Module):
         E, top = int(r["experts"]), int(r["top"])
         if not 1 <= top <= E:
             raise ValueError(f"{prefix}: top {top} of {E} experts")
-        self.router = ReplicatedLinear(width, E, bias=True, params_dtype=torch.float32, prefix=f"{prefix}.router")
+        sh = spec.get("shared")
+        self.num_experts = E
+        # one fp32 product for everything that is a dot product with x in 32 bits: the router's rows and, last, the
+        # shared expert's gate
+        rows = E + (1 if sh else 0)
+        self.route_weight = nn.Parameter(torch.zeros((rows, width), dtype=torch.float32), requires_grad=False)
+        self.route_bias = nn.Parameter(torch.zeros((rows,), dtype=torch.float32), requires_grad=False)
+
+        def load_rows(param, t, part=0):
+            lo, hi = (0, E) if part == 0 else (E, rows)
+            param.data[lo:hi].copy_(t.to(torch.float32).reshape(param.data[lo:hi].shape))
+        set_weight_attrs(self.route_weight, {"weight_loader": load_rows})
+        set_weight_attrs(self.route_bias, {"weight_loader": load_rows})
         self.experts = FusedMoE(E, top, width, int(ex["ff"]), renormalize=True, quant_config=quant_config,
                                 prefix=f"{prefix}.experts", activation=ACT, gated=False)
-        sh = spec.get("shared")
         self.shared = SquaredReluMLP(width, int(sh["ff"]), quant_config, f"{prefix}.shared") if sh else None
-        if sh:
-            self.shared_gate = _fp32_param((width,), 0.0)
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
-        xf = x.float()
-        logits = F.linear(xf, self.router.weight, self.router.bias)           # the router runs in fp32
-        out = self.experts(x, logits)
-        if self.shared is not None:
-            g = torch.sigmoid(xf @ self.shared_gate).unsqueeze(1)
-            out = torch.addcmul(out.float(), self.shared(x).float(), g).to(x.dtype)
-        return out
+    def forward(self, x: torch.Tensor):
+        """Returns (routed experts' sum, shared expert's output or None, its gate's logit fp32 [T, 1] or None); the
+        caller's residual pass forms routed + shared * sigmoid(gate)."""
+        z = ops.fp32_rows_dot(x, self.route_weight, self.route_bias)           # fp32 logits [T, E (+ 1)]
+        out = self.experts(x, z[:, : self.num_experts])
+        if self.shared is None:
+            return out, None, None
+        return out, self.shared(x), z[:, self.num_experts:]
 
 
 class LayerNormParams(nn.Module):
@@ -165,6 +173,7 @@ class SevazenBlock(nn.Module):
         self.mixer = make_mixer(spec["type"], spec["mixer"], width, eps, users, quant_config, f"{prefix}.mixer")
         mlp = spec.get("mlp")
         self.has_mlp = mlp is not None
+        self.routed = self.has_mlp and mlp.get("kind", "dense") != "dense"
         if self.has_mlp:
             self.norm2 = LayerNormParams(width)
             if mlp.get("kind", "dense") == "dense":
@@ -178,8 +187,8 @@ class SevazenBlock(nn.Module):
         y = self.mixer(h, positions, user)
         h = ops.residual_layer_norm(x, y, self.norm1.weight, self.norm1.bias, self.eps, y.dtype)
         if self.has_mlp:
-            y = self.mlp(h)
-            h = ops.residual_layer_norm(x, y, self.norm2.weight, self.norm2.bias, self.eps, y.dtype)
+            y, y2, gate = self.mlp(h) if self.routed else (self.mlp(h), None, None)
+            h = ops.residual_layer_norm(x, y, self.norm2.weight, self.norm2.bias, self.eps, y.dtype, y2, gate)
         return h
 
 
@@ -261,15 +270,15 @@ class SevazenForCausalLM(nn.Module):
             if isinstance(blk.mlp, SquaredReluMLP):
                 return (f"{base}mlp.{self._FF[leaf]}", None, None) if leaf in self._FF else None
             if leaf == "router":
-                return f"{base}mlp.router.weight", None, None
+                return f"{base}mlp.route_weight", 0, None
             if leaf == "router.b":
-                return f"{base}mlp.router.bias", None, None
+                return f"{base}mlp.route_bias", 0, None
             sub, _, w = leaf.partition(".")
             if sub == "shared" and blk.mlp.shared is not None:
                 if w in self._FF:
                     return f"{base}mlp.shared.{self._FF[w]}", None, None
                 if w == "sg":
-                    return f"{base}mlp.shared_gate", None, None
+                    return f"{base}mlp.route_weight", 1, None
             em = re.fullmatch(r"e(\d+)", sub)
             if em and w in self._EXPERT and int(em.group(1)) < blk.mlp.experts.global_num_experts:
                 t, shard = self._EXPERT[w]

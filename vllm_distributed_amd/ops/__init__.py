@@ -907,8 +907,8 @@ def group_rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, groups: in
     return out
 
 
-def moe_grouped_ok(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor) -> bool:
-    I = w13.shape[1] // 2
+def moe_grouped_ok(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, gated: bool = True) -> bool:
+    I = w13.shape[1] // 2 if gated else w13.shape[1]
     return (x.dtype in (torch.bfloat16, torch.float16) and w13.shape[2] % 128 == 0 and I % 128 == 0
             and w2.shape[1] % 16 == 0 and w13.dtype in (x.dtype, torch.float8_e4m3fn) and w13.dtype == w2.dtype
             and w13.shape[0] <= 1024)
@@ -1162,6 +1162,30 @@ def _moe_pairs(x, w13, w2, topk_w, topk_ids, activation: str, act_limit: float, 
     return out
 
 
+def _moe_grouped_ungated(x, w1, w2, topk_w, topk_ids, activation: str):
+    """Few pairs (decoding): experts without a gate half through the grouped skinny MFMA GEMMs, weights streamed once."""
+    T, H = x.shape
+    k = topk_ids.shape[1]
+    E, I, _ = w1.shape
+    dev = x.device
+    ids, tw = topk_ids.contiguous(), topk_w.contiguous()
+    sorted_ids = torch.empty(T * k, dtype=torch.int32, device=dev)
+    offsets = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    st = N.stream()
+    N.call("vda_moe_align", sorted_ids.data_ptr(), offsets.data_ptr(), ids.data_ptr(), T * k, E, st)
+    inter = torch.empty((T * k, I), dtype=x.dtype, device=dev)
+    out2 = torch.empty((T * k, H), dtype=x.dtype, device=dev)
+    out = torch.empty((T, H), dtype=x.dtype, device=dev)
+    N.call("vda_moe_up_act", inter.data_ptr(), x.data_ptr(), w1.data_ptr(), sorted_ids.data_ptr(), offsets.data_ptr(),
+           E, I, H, k, T, x.stride(0), N.dt(x.dtype), int(moe_rows_form(T * k, E, I, w1.element_size())),
+           N.ACT[activation], st)
+    N.call("vda_moe_down", out2.data_ptr(), inter.data_ptr(), w2.data_ptr(), None, tw.data_ptr(),
+           sorted_ids.data_ptr(), offsets.data_ptr(), E, H, I, T, N.dt(x.dtype), N.dt(w2.dtype),
+           int(moe_rows_form(T * k, E, H, w2.element_size())), st)
+    N.call("vda_moe_sum", out.data_ptr(), out2.data_ptr(), ids.data_ptr(), T, H, k, out.stride(0), N.dt(x.dtype), st)
+    return out
+
+
 MOE_ACTIVATIONS = ("silu", "gelu", "gelu_tanh", "gelu_pytorch_tanh", "relu", "relu2", "clamped_swiglu")
 
 
@@ -1182,6 +1206,9 @@ def fused_moe(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, topk_w: torc
     if not gated:
         if activation == "clamped_swiglu" or w13_scale is not None or w2_scale is not None or x_scale is not None:
             raise ValueError("experts without a gate half take an element-wise activation and unquantised weights")
+        if _dev(x) and moe_grouped_ok(x, w13, w2, gated=False) and w13.dtype == x.dtype and (
+                x.shape[0] * topk_ids.shape[1] <= envs.VDA_MOE_GROUPED_MAX_PAIRS or not moe_tiled_ok(x, w13, w2, False)):
+            return _moe_grouped_ungated(_contig_last(x), w13, w2, topk_w, topk_ids, activation)
         if _dev(x) and moe_tiled_ok(x, w13, w2, gated=False):
             return _moe_tiled(_contig_last(x), w13, w2, topk_w, topk_ids, None, None, False, activation, gated=False)
         if _dev(x) and moe_pairs_ok(x, w13, w2, gated=False):
@@ -1564,15 +1591,31 @@ def mlstm(proj: torch.Tensor, i_bias: torch.Tensor, f_bias: torch.Tensor, norm_w
 
 
 # ---- fp32 residual with a layer norm on every sub-layer's output ------------------------------------------------
+def fp32_rows_dot(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Dot products a design wants in fp32 whatever the activations' type: x [T, W] against fp32 rows weight [R, W]
+    (+ bias [R]) -> fp32 [T, R] (router logits, one-number gates), one launch without a widened copy of x."""
+    if not _dev(x) or weight.shape[0] > 256:
+        return R.fp32_rows_dot(x, weight, bias)
+    assert x.stride(1) == 1 and weight.dtype == torch.float32 and weight.is_contiguous()
+    assert bias is None or (bias.dtype == torch.float32 and bias.is_contiguous())
+    T, W = x.shape
+    out = torch.empty((T, weight.shape[0]), dtype=torch.float32, device=x.device)
+    N.call("vda_fp32_rows_dot", out.data_ptr(), x.data_ptr(), x.stride(0), weight.data_ptr(), N.ptr(bias), T,
+           weight.shape[0], W, N.dt(x.dtype), N.stream())
+    return out
+
+
 def residual_layer_norm(x: torch.Tensor, y: Optional[torch.Tensor], weight: torch.Tensor,
-                        bias: Optional[torch.Tensor], eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+                        bias: Optional[torch.Tensor], eps: float, out_dtype: torch.dtype,
+                        y2: Optional[torch.Tensor] = None, y2_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """One pass over the fp32 residual ``x`` [T, W].  With ``y`` (a sub-layer's output): x += layer_norm(y) * weight +
     bias, in place, and the updated x is returned in ``out_dtype`` (x itself when that is fp32): the next sub-layer
     reads the residual as it is.  Without ``y``: layer_norm(x) * weight + bias in ``out_dtype``; x stays.
-    Weight and bias are fp32 [W]."""
+    Weight and bias are fp32 [W].  ``y2`` [T, W] with ``y2_gate`` fp32 [T, 1] (row stride arbitrary): the sub-layer's
+    output is y + y2 * sigmoid(y2_gate), formed inside the same pass (a shared expert behind its gate)."""
     T, W = x.shape
     if not _dev(x) or W * 4 > 60 * 1024:
-        return R.residual_layer_norm(x, y, weight, bias, eps, out_dtype)
+        return R.residual_layer_norm(x, y, weight, bias, eps, out_dtype, y2, y2_gate)
     assert x.dtype == torch.float32 and x.is_contiguous() and weight.dtype == torch.float32
     assert bias is None or bias.dtype == torch.float32
     h = None
@@ -1580,8 +1623,13 @@ def residual_layer_norm(x: torch.Tensor, y: Optional[torch.Tensor], weight: torc
         h = torch.empty((T, W), dtype=out_dtype, device=x.device)
     if y is not None:
         assert y.stride(1) == 1 and y.shape == (T, W) and y.dtype == out_dtype
+    if y2 is not None:
+        assert y is not None and y2.shape == (T, W) and y2.dtype == y.dtype and y2.stride(1) == 1
+        assert y2_gate.dtype == torch.float32 and y2_gate.shape[0] == T
     N.call("vda_residual_layer_norm", x.data_ptr(), N.ptr(y), y.stride(0) if y is not None else 0, weight.data_ptr(),
-           N.ptr(bias), N.ptr(h), W, float(eps), T, W, N.dt(out_dtype), N.stream())
+           N.ptr(bias), N.ptr(h), W, float(eps), T, W, N.dt(out_dtype), N.ptr(y2),
+           y2.stride(0) if y2 is not None else 0, N.ptr(y2_gate), y2_gate.stride(0) if y2_gate is not None else 0,
+           N.stream())
     return h if h is not None else x
 
 

@@ -269,7 +269,7 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
   for (int mt = 0; mt < 4; ++mt) {
     const int i = mt * 16 + r;
     pid[mt] = i < cnt ? sorted[beg + i] : -1;
-    const int row = pid[mt] < 0 ? 0 : (GATE_UP ? pid[mt] / top_k : pid[mt]);
+    const int row = pid[mt] < 0 ? 0 : pid[mt] / top_k;        // the down form passes top_k = 1
     xp[mt] = act + (long)row * act_stride;
   }
   f32x4 acc0[4], acc1[4];
@@ -322,9 +322,10 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
           o[i] = (T)gated_pair(gte, up, act_kind, act_limit);
         }
       } else {
-        const float tw = topk_w[pid[mt]] * ws;
+        // down form: times the routing weight; first GEMM of experts without a gate half: act(v), no weight
+        const float tw = (topk_w ? topk_w[pid[mt]] : 1.f) * ws;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) o[i] = (T)(a[i] * tw);
+        for (int i = 0; i < 4; ++i) o[i] = (T)(act_kind >= 0 ? gate_act(a[i] * tw, act_kind) : a[i] * tw);
       }
       *reinterpret_cast<V4*>(out + (long)pid[mt] * out_stride + n0 + 4 * g) = o;
     }
@@ -377,7 +378,7 @@ __global__ __launch_bounds__(256) void moe_grouped_rows_kernel(
   for (int i = 0; i < MT; ++i) {
     const int t = (tid >> 4) + 16 * i;
     const int id = t < cnt ? sorted[beg + t] : -1;
-    xrow[i] = id < 0 ? nullptr : act + (long)(GATE_UP ? id / top_k : id) * act_stride + piece * 8;
+    xrow[i] = id < 0 ? nullptr : act + (long)(id / top_k) * act_stride + piece * 8;       // down form: top_k = 1
   }
   int pid[MT];
 #pragma unroll
@@ -451,9 +452,9 @@ __global__ __launch_bounds__(256) void moe_grouped_rows_kernel(
           o[i] = (T)gated_pair(gte, up, act_kind, act_limit);
         }
       } else {
-        const float tw = topk_w[pid[mt]] * ws;
+        const float tw = (topk_w ? topk_w[pid[mt]] : 1.f) * ws;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) o[i] = (T)(acc0[mt][i] * tw);
+        for (int i = 0; i < 4; ++i) o[i] = (T)(act_kind >= 0 ? gate_act(acc0[mt][i] * tw, act_kind) : acc0[mt][i] * tw);
       }
       *reinterpret_cast<V4*>(out + (long)pid[mt] * out_stride + n0 + 4 * g) = o;
     }
@@ -495,13 +496,37 @@ VDA_EXPORT int vda_moe_down(void* out2, const void* inter, const void* w2, const
   dim3 grid(rows ? H / 64 : H / 16, E, (max_pairs + per - 1) / per), block(256);
   const long es = (long)H * I;
 #define L(TT, WL) do { if (rows && per == 128) hipLaunchKernelGGL((moe_grouped_rows_kernel<TT, WL, false, 8>), grid, block, 0, st, \
-        (TT*)out2, (const TT*)inter, w2, w_scale, topk_w, sorted, offsets, H, I, 1, (long)I, (long)H, es, 0, 0.f); \
+        (TT*)out2, (const TT*)inter, w2, w_scale, topk_w, sorted, offsets, H, I, 1, (long)I, (long)H, es, -1, 0.f); \
     else if (rows) hipLaunchKernelGGL((moe_grouped_rows_kernel<TT, WL, false, 4>), grid, block, 0, st, (TT*)out2, \
-        (const TT*)inter, w2, w_scale, topk_w, sorted, offsets, H, I, 1, (long)I, (long)H, es, 0, 0.f); \
+        (const TT*)inter, w2, w_scale, topk_w, sorted, offsets, H, I, 1, (long)I, (long)H, es, -1, 0.f); \
     else hipLaunchKernelGGL((moe_grouped_kernel<TT, WL, false>), grid, block, 0, st, (TT*)out2, (const TT*)inter, \
-        w2, w_scale, topk_w, sorted, offsets, H, I, 1, (long)I, (long)H, es, 0, 0.f); } while (0)
+        w2, w_scale, topk_w, sorted, offsets, H, I, 1, (long)I, (long)H, es, -1, 0.f); } while (0)
   if (dtype == VDA_BF16) { if (wdtype == VDA_FP8) L(bf16_t, WLoadFp8<bf16_t>); else L(bf16_t, WLoad<bf16_t>); }
   else if (dtype == VDA_F16) { if (wdtype == VDA_FP8) L(f16_t, WLoadFp8<f16_t>); else L(f16_t, WLoad<f16_t>); }
+  else return -3;
+#undef L
+  VDA_CHECK_LAUNCH();
+  return 0;
+}
+
+// First GEMM of experts without a gate half: inter[p, :] = act(x[p / top_k] . W1_e^T), W1 [E, I, K].  The grouped
+// skinny kernels in their single-accumulator form, rows gathered per pair, the activation in the epilogue.
+VDA_EXPORT int vda_moe_up_act(void* inter, const void* x, const void* w1, const int* sorted, const int* offsets, int E,
+                              int I, int K, int top_k, int max_pairs, long x_stride, int dtype, int rows_form,
+                              int act_kind, hipStream_t st) {
+  if (I % 16 || K % 128 || E < 1 || max_pairs < 1 || top_k < 1 || act_kind < 0) return -1;
+  const bool rows = rows_form && I % 64 == 0;
+  const int per = rows && rows_form == 2 ? 128 : 64;
+  dim3 grid(rows ? I / 64 : I / 16, E, (max_pairs + per - 1) / per), block(256);
+  const long es = (long)I * K;
+#define L(TT, WL) do { if (rows && per == 128) hipLaunchKernelGGL((moe_grouped_rows_kernel<TT, WL, false, 8>), grid, block, 0, st, \
+        (TT*)inter, (const TT*)x, w1, (const float*)nullptr, (const float*)nullptr, sorted, offsets, I, K, top_k, x_stride, (long)I, es, act_kind, 0.f); \
+    else if (rows) hipLaunchKernelGGL((moe_grouped_rows_kernel<TT, WL, false, 4>), grid, block, 0, st, (TT*)inter, \
+        (const TT*)x, w1, (const float*)nullptr, (const float*)nullptr, sorted, offsets, I, K, top_k, x_stride, (long)I, es, act_kind, 0.f); \
+    else hipLaunchKernelGGL((moe_grouped_kernel<TT, WL, false>), grid, block, 0, st, (TT*)inter, (const TT*)x, \
+        w1, (const float*)nullptr, (const float*)nullptr, sorted, offsets, I, K, top_k, x_stride, (long)I, es, act_kind, 0.f); } while (0)
+  if (dtype == VDA_BF16) L(bf16_t, WLoad<bf16_t>);
+  else if (dtype == VDA_F16) L(f16_t, WLoad<f16_t>);
   else return -3;
 #undef L
   VDA_CHECK_LAUNCH();

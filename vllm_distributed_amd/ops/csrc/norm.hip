@@ -317,30 +317,54 @@ VDA_EXPORT int vda_residual_norms(float* x, const void* y, long y_stride, const 
 // fp32 residual whose sub-layers are normed on their OUTPUT: x += (y - mean(y)) / sqrt(var(y) + eps) * w + b, in place,
 // and the updated row goes out once more in the activation type, as the next sub-layer's input (one launch for the
 // norm, the residual sum and the cast).  Without y: h = layer norm of x itself (the model's last norm), x stays.
+// With y2 and gate the sub-layer's output is y + y2 * sigmoid(gate[t]) (a shared expert behind its gate), formed here.
 // The source row sits in LDS between the passes (mean, squared deviations, output).
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void residual_layer_norm_kernel(float* __restrict__ x, const T* __restrict__ y,
                                                                   long y_stride, const float* __restrict__ w,
                                                                   const float* __restrict__ b, T* __restrict__ h,
-                                                                  long h_stride, float eps, int W) {
+                                                                  long h_stride, float eps, int W,
+                                                                  const T* __restrict__ y2, long y2_stride,
+                                                                  const float* __restrict__ gate, long gate_stride) {
+  // VEC consecutive values per thread and trip (4: rows whose width and strides are multiples of four, moved as
+  // 16-byte fp32 / 8- or 16-byte activation vectors)
+  using V4 = typename Vec<T>::v4;
   extern __shared__ float row[];
   __shared__ float red[16];
   const long t = blockIdx.x;
   const int tid = threadIdx.x;
   float* xr = x + t * W;
   const T* yr = y ? y + t * y_stride : nullptr;
+  // a second part of the sub-layer's output behind a sigmoid gate of one number per row: y + y2 * sigmoid(gate[t])
+  const T* y2r = (y && y2) ? y2 + t * y2_stride : nullptr;
+  const float g2 = y2r ? 1.f / (1.f + expf(-gate[t * gate_stride])) : 0.f;
   float s = 0.f;
   for (int c = tid * VEC; c < W; c += 256 * VEC) {
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) {
-      const float v = yr ? (float)yr[c + i] : xr[c + i];
-      row[c + i] = v;
-      s += v;
+    float v[VEC];
+    if (VEC == 4) {
+      if (yr) {
+        const V4 q = *reinterpret_cast<const V4*>(yr + c);
+        v[0] = (float)q[0]; v[1 % VEC] = (float)q[1]; v[2 % VEC] = (float)q[2]; v[3 % VEC] = (float)q[3];
+        if (y2r) {
+          const V4 q2 = *reinterpret_cast<const V4*>(y2r + c);
+          v[0] += g2 * (float)q2[0]; v[1 % VEC] += g2 * (float)q2[1]; v[2 % VEC] += g2 * (float)q2[2];
+          v[3 % VEC] += g2 * (float)q2[3];
+        }
+      } else {
+        const f32x4 q = *reinterpret_cast<const f32x4*>(xr + c);
+        v[0] = q[0]; v[1 % VEC] = q[1]; v[2 % VEC] = q[2]; v[3 % VEC] = q[3];
+      }
+      *reinterpret_cast<f32x4*>(row + c) = f32x4{v[0], v[1 % VEC], v[2 % VEC], v[3 % VEC]};
+    } else {
+      v[0] = yr ? (float)yr[c] + (y2r ? g2 * (float)y2r[c] : 0.f) : xr[c];
+      row[c] = v[0];
     }
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) s += v[i];
   }
   const float mean = block_sum(s, red) / (float)W;
   float ss = 0.f;
-  for (int c = tid * VEC; c < W; c += 256 * VEC) {
+  for (int c = tid * VEC; c < W; c += 256 * VEC) {       // a thread re-reads what it wrote itself
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
       const float d = row[c + i] - mean;
@@ -349,27 +373,41 @@ __global__ __launch_bounds__(256) void residual_layer_norm_kernel(float* __restr
   }
   const float r = 1.f / sqrtf(block_sum(ss, red) / (float)W + eps);
   for (int c = tid * VEC; c < W; c += 256 * VEC) {
+    float v[VEC];
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) {
-      float v = (row[c + i] - mean) * r * w[c + i] + (b ? b[c + i] : 0.f);
+    for (int i = 0; i < VEC; ++i) v[i] = (row[c + i] - mean) * r * w[c + i] + (b ? b[c + i] : 0.f);
+    if (VEC == 4) {
       if (yr) {
-        v += xr[c + i];
-        xr[c + i] = v;
+        const f32x4 q = *reinterpret_cast<const f32x4*>(xr + c);
+        v[0] += q[0]; v[1 % VEC] += q[1]; v[2 % VEC] += q[2]; v[3 % VEC] += q[3];
+        *reinterpret_cast<f32x4*>(xr + c) = f32x4{v[0], v[1 % VEC], v[2 % VEC], v[3 % VEC]};
       }
-      if (h) h[t * h_stride + c + i] = (T)v;
+      if (h) {
+        V4 o;
+        o[0] = (T)v[0]; o[1] = (T)v[1 % VEC]; o[2] = (T)v[2 % VEC]; o[3] = (T)v[3 % VEC];
+        *reinterpret_cast<V4*>(h + t * h_stride + c) = o;
+      }
+    } else {
+      if (yr) {
+        v[0] += xr[c];
+        xr[c] = v[0];
+      }
+      if (h) h[t * h_stride + c] = (T)v[0];
     }
   }
 }
 
 VDA_EXPORT int vda_residual_layer_norm(float* x, const void* y, long y_stride, const float* w, const float* b,
-                                       void* h, long h_stride, float eps, int T, int W, int dtype, hipStream_t st) {
+                                       void* h, long h_stride, float eps, int T, int W, int dtype, const void* y2,
+                                       long y2_stride, const float* gate, long gate_stride, hipStream_t st) {
   if (T <= 0) return 0;
-  if (!w || (!y && !h)) return -1;
+  if (!w || (!y && !h) || (y2 && (!y || !gate))) return -1;
   const size_t lds = (size_t)W * 4;
   if (lds > 60 * 1024) return -2;
-  const bool vec = W % 4 == 0 && y_stride % 4 == 0 && h_stride % 4 == 0;
+  const bool vec = W % 4 == 0 && y_stride % 4 == 0 && h_stride % 4 == 0 && y2_stride % 4 == 0;
 #define L2(TT, VV) hipLaunchKernelGGL((residual_layer_norm_kernel<TT, VV>), dim3(T), dim3(256), lds, st, x,          \
-                                      (const TT*)y, y_stride, w, b, (TT*)h, h_stride, eps, W)
+                                      (const TT*)y, y_stride, w, b, (TT*)h, h_stride, eps, W, (const TT*)y2,          \
+                                      y2_stride, gate, gate_stride)
 #define L(TT) do { if (vec) L2(TT, 4); else L2(TT, 1); } while (0)
   if (dtype == VDA_BF16) L(bf16_t);
   else if (dtype == VDA_F16) L(f16_t);
@@ -377,6 +415,38 @@ VDA_EXPORT int vda_residual_layer_norm(float* x, const void* y, long y_stride, c
   else return -3;
 #undef L
 #undef L2
+  VDA_CHECK_LAUNCH();
+  return 0;
+}
+
+// Dot products that a design wants in fp32 although the activations are 16-bit: out[t, r] = bias[r] + x[t, :] . w[r, :]
+// with fp32 weights (router logits, one-number gates).  One workgroup per token, a wave per output row in turn.
+template <typename T>
+__global__ __launch_bounds__(256) void fp32_rows_dot_kernel(float* __restrict__ out, const T* __restrict__ x,
+                                                            long x_stride, const float* __restrict__ w,
+                                                            const float* __restrict__ bias, int R, int W) {
+  const long t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const T* xr = x + t * x_stride;
+  for (int r = wave; r < R; r += 4) {
+    const float* wr = w + (long)r * W;
+    float a = 0.f;
+    for (int c = lane; c < W; c += 64) a += (float)xr[c] * wr[c];
+    a = wave_sum(a);
+    if (lane == 0) out[t * R + r] = a + (bias ? bias[r] : 0.f);
+  }
+}
+
+VDA_EXPORT int vda_fp32_rows_dot(float* out, const void* x, long x_stride, const float* w, const float* bias, int T,
+                                 int R, int W, int dtype, hipStream_t st) {
+  if (T <= 0 || R <= 0) return 0;
+#define L(TT) hipLaunchKernelGGL((fp32_rows_dot_kernel<TT>), dim3(T), dim3(256), 0, st, out, (const TT*)x, x_stride, \
+                                 w, bias, R, W)
+  if (dtype == VDA_BF16) L(bf16_t);
+  else if (dtype == VDA_F16) L(f16_t);
+  else if (dtype == VDA_F32) L(float);
+  else return -3;
+#undef L
   VDA_CHECK_LAUNCH();
   return 0;
 }

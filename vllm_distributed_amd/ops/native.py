@@ -66,12 +66,14 @@ _SIGS = {
     "vda_moe_grouped_sigmoid_topk": [P, P, P, P, I, I, I, I, I, I, L, I, P],
     "vda_group_rms_norm": [P, L, P, L, P, F, I, I, I, I, I, P],
     "vda_moe_pairs": [P, L, P, P, L, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
-    "vda_residual_layer_norm": [P, P, L, P, P, P, L, F, I, I, I, P],
+    "vda_residual_layer_norm": [P, P, L, P, P, P, L, F, I, I, I, P, L, P, L, P],
+    "vda_fp32_rows_dot": [P, P, L, P, P, I, I, I, I, P],
     "vda_qk_norm_rope_cache": [P, P, L, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, I, I, P],
     "vda_map_combine": [P, P, P, P, L, I, I, I, I, I, F, F, I, P],
     "vda_masked_softmax_attention": [P, P, P, P, P, L, P, P, P, P, P, L, F, I, I, I, F, F, I, I, I, I, I, I, I, I, P],
     "vda_moe_gate_up": [P, P, P, P, P, P, I, I, I, I, I, L, I, I, I, I, F, P],
     "vda_moe_down": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
+    "vda_moe_up_act": [P, P, P, P, P, I, I, I, I, I, L, I, I, I, P],
     "vda_moe_sum": [P, P, P, I, I, I, L, I, P],
     "vda_ep_prep": [P, I, I, I, P, P, P, P, P, P],
     "vda_moe_tile_map": [P, P, P, P, P, I, I, I, P],

@@ -806,11 +806,13 @@ def mlstm(proj, i_bias, f_bias, norm_w, state_nm, state_s, qsl, seq_lens, slot_t
 
 
 # ---- fp32 residual with a layer norm on every sub-layer's output -------------------------------------------------
-def residual_layer_norm(x, y, weight, bias, eps: float, out_dtype):
+def residual_layer_norm(x, y, weight, bias, eps: float, out_dtype, y2=None, y2_gate=None):
     """x fp32 [T, W].  With ``y`` (a sub-layer's output): x += (y - mean) / sqrt(var + eps) * weight + bias, in place, and
     x comes back in ``out_dtype`` (the next sub-layer reads the residual itself).  Without: the layer norm of x comes
-    back in ``out_dtype`` and x stays."""
+    back in ``out_dtype`` and x stays.  ``y2`` / ``y2_gate`` [T, 1]: the sub-layer's output is y + y2 * sigmoid(gate)."""
     src = y.float() if y is not None else x
+    if y2 is not None:
+        src = src + y2.float() * torch.sigmoid(y2_gate.float().reshape(-1, 1))
     mu = src.mean(-1, keepdim=True)
     d = src - mu
     n = d * torch.rsqrt(d.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
@@ -911,3 +913,9 @@ def masked_softmax_attention(qn, k_cache, v_cache, block_table, seq_lens, qsl, s
     if gate is not None:
         out = out * torch.sigmoid(gate[:T].float())
     return out.to(out_dtype)
+
+
+def fp32_rows_dot(x, weight, bias):
+    """x [T, W] (any type) against fp32 rows weight [R, W] (+ bias [R]) in fp32: [T, R]."""
+    out = x.float() @ weight.float().t()
+    return out + bias.float() if bias is not None else out
