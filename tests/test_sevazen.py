@@ -263,12 +263,20 @@ def test_masked_attention_paged(dev, dt, H, G, D, E, maps, window, chunk, sink, 
     if mfma:
         # the matrix-core kernels: the decoded token through the decode form (whole, and with its keys dealt to three
         # workgroups), the portion and the prompt through the tiled form
-        got = [ops.masked_softmax_attention_mfma(qn, kc, vc, table.to(dev), sl, qsl, qsl[1:] - 1, 1, 1, 2, sum(news[1:]),
-                                                 1, splits, max(news), scale, H, window, chunk,
-                                                 sk.to(dev) if sink else None, maps, lam, eps, out_scale, gt)
-               for splits in (1, 3)]
-        assert rel(got[1], got[0]) < 1e-2
-        got = got[0]
+        def run(splits):
+            return ops.masked_softmax_attention_mfma(qn, kc, vc, table.to(dev), sl, qsl, qsl[1:] - 1, 1, 1, 2,
+                                                     sum(news[1:]), 1, splits, max(news), scale, H, window, chunk,
+                                                     sk.to(dev) if sink else None, maps, lam, eps, out_scale, gt)
+        got = run(1)
+        assert rel(run(3), got) < 1e-2
+        if D == 128:                                  # the 8-wave form for prompts, whenever the shape allows
+            from vllm_distributed_amd.ops import native
+            native.call("vda_set_prefill_variant", 3)
+            try:
+                wide = run(1)
+            finally:
+                native.call("vda_set_prefill_variant", 1)
+            assert rel(wide, want) < OP_TOL[dt] * 3
     else:
         got = ops.masked_softmax_attention(qn, kc, vc, table.to(dev), sl, qsl, scale, window, chunk,
                                            sk.to(dev) if sink else None, maps, lam, eps, out_scale, gt, max(news), dt)

@@ -198,7 +198,8 @@ class SevazenForCausalLM(nn.Module):
     # convolution states live in per-row slots beside the paged keys and values
     row_state_slots = True
     # kernels outside the common set that this model launches (ops/build.py builds them on first use)
-    native_sources = ("masked_attention.hip", "mamba.hip", "moe.hip", "gemm_tile.hip")
+    native_sources = ("masked_attention.hip", "attention.hip", "attention_prefill.hip", "mamba.hip", "moe.hip",
+                      "gemm_tile.hip")
 
     def __init__(self, vllm_config: VllmConfig, prefix: str = ""):
         super().__init__()

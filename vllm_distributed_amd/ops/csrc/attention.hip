@@ -835,7 +835,7 @@ VDA_EXPORT int vda_paged_attention_prefill(
   if (G > 128) return -4;
   if (!causal && (window > 0 || chunk > 0)) return -5;
   if (chunk < 0 || v_shift < 0 || (Hkv >> v_shift) << v_shift != Hkv) return -7;
-  const bool extras = sink != nullptr || chunk > 0 || v_shift > 0;     // served by the 4-wave form only
+  const bool extras = sink != nullptr || chunk > 0 || v_shift > 0;     // not in the direct-to-register form
   const int q_tile = 128 / G;     // 4 waves x 32 columns
   AttnParams p{q, k_cache, v_cache, out, nullptr, nullptr, block_table, seq_lens, q_start_loc, alibi,
                num_seqs, Hq, Hkv, max_blocks, 1, q_stride, out_stride, scale * (kv_fp8 ? k_scale : 1.f), softcap,
@@ -843,7 +843,7 @@ VDA_EXPORT int vda_paged_attention_prefill(
   p.sink = sink; p.chunk = chunk; p.v_shift = v_shift;
   // Wide form (8 waves, 256 columns, 64-key tiles): head size 128 and enough query tiles to occupy the
   // chip (one workgroup per CU); short chunks keep the 4-wave form, which cuts them into more workgroups.
-  if (!extras && D == 128 && 256 % G == 0 && (g_prefill_variant == 1 || g_prefill_variant == 3)) {
+  if (D == 128 && 256 % G == 0 && (g_prefill_variant == 1 || g_prefill_variant == 3)) {
     const int wide_tile = 256 / G;
     const long wgs = (long)(num_tokens / wide_tile) * Hkv;
     if (g_prefill_variant == 3 || wgs >= g_prefill_wide_min_wgs) {

@@ -123,7 +123,8 @@ __global__ __launch_bounds__(512) void paged_prefill_wide_kernel(AttnParams p, i
   const bool valid = qt < qt_end;
   const int head = kvh * G + hq;
   const int limit = valid ? (p.causal ? ctx + qt + 1 : seq_len) : 0;
-  const int lower = (valid && p.window > 0) ? max(0, limit - p.window) : 0;
+  int lower = (valid && p.window > 0) ? max(0, limit - p.window) : 0;
+  if (valid && p.chunk > 0) lower = max(lower, (limit - 1) / p.chunk * p.chunk);     // keys of the query's chunk only
   const float slope = (p.alibi && valid) ? p.alibi[head] : 0.f;
   const long col_off = valid ? (long)(qs + qt) : -1;
   V8 qf[8];
@@ -143,13 +144,15 @@ __global__ __launch_bounds__(512) void paged_prefill_wide_kernel(AttnParams p, i
   }
   // workgroup-uniform key range (all waves take part in every tile copy)
   const int wg_hi = p.causal ? ctx + qt_end : seq_len;
-  const int wg_lo = p.window > 0 ? max(0, ctx + q0 + 1 - p.window) : 0;
+  int wg_lo = p.window > 0 ? max(0, ctx + q0 + 1 - p.window) : 0;
+  if (p.chunk > 0 && p.causal) wg_lo = max(wg_lo, (ctx + q0) / p.chunk * p.chunk);
   const int kt_lo = wg_lo / KT, kt_hi = (wg_hi + KT - 1) / KT;
 
   const CT* kc = (const CT*)p.k_cache;
   const CT* vc = (const CT*)p.v_cache;
-  const unsigned blk_stride = (unsigned)p.Hkv * BS * D;          // elements per cache block (K and V alike)
-  const unsigned k_head = (unsigned)kvh * BS * D, v_head = (unsigned)kvh * D * BS;
+  const unsigned blk_stride = (unsigned)p.Hkv * BS * D;          // elements per K cache block
+  const unsigned v_blk_stride = (unsigned)(p.Hkv >> p.v_shift) * D * BS;     // per V cache block (fewer heads when shared)
+  const unsigned k_head = (unsigned)kvh * BS * D, v_head = (unsigned)(kvh >> p.v_shift) * D * BS;
 
   // ---- copy step: 1024 K pieces and 1024 V pieces of 16 bytes per tile, two of each per thread ----
   // K piece pi: key = pi >> 4, piece = pi & 15.   V piece pi: cache block j = pi / (128 * PPB) of the tile,
@@ -184,7 +187,7 @@ __global__ __launch_bounds__(512) void paged_prefill_wide_kernel(AttnParams p, i
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       rk[i] = KVLoad<T, F8>::ld(kc + (size_t)(unsigned)kblk[i] * blk_stride + k_src[i]);
-      rv[i] = KVLoad<T, F8>::ld(vc + (size_t)(unsigned)vblk[i] * blk_stride + v_src[i]);
+      rv[i] = KVLoad<T, F8>::ld(vc + (size_t)(unsigned)vblk[i] * v_blk_stride + v_src[i]);
     }
   };
   auto sstore = [&](int buf) {
@@ -208,6 +211,10 @@ __global__ __launch_bounds__(512) void paged_prefill_wide_kernel(AttnParams p, i
   for (int t = 0; t < 4; ++t) v_rd[t] = c32 * 128 + 16 * ((2 * t + hi) ^ ((c32 >> 1) & 7));
 
   float m = -INFINITY, l = 0.f;       // l: this lane's half of the column's sum
+  if (p.sink && valid) {               // a sink: the maximum starts there, the sum with its weight of one (in one half)
+    m = p.sink[head] * 1.4426950408889634f;
+    l = hi == 0 ? 1.f : 0.f;
+  }
   f32x16 acc[4];
 #pragma unroll
   for (int db = 0; db < 4; ++db)

@@ -83,12 +83,102 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_kernel(
   }
 }
 
+// The same with 8 consecutive values per lane (16-byte accesses for 16-bit rows): LPU = D / 8 lanes share a unit, so a
+// workgroup takes 256 / LPU units at a time; the pair partner of a lane's values sits in the lane rot / 16 further on
+// (or back) and arrives by a shuffle.  For D in {32, 64, 128, 256}, rot / 2 a multiple of 8, rows 16-byte aligned.
+template <typename T, int LPU>
+__global__ __launch_bounds__(256) void qk_norm_rope_cache_vec_kernel(
+    T* __restrict__ qn, const T* __restrict__ qkv, long qkv_stride, const float* __restrict__ q_w,
+    const float* __restrict__ k_w, const float* __restrict__ cos_sin, const long* __restrict__ positions,
+    T* __restrict__ k_cache, T* __restrict__ v_cache, const long* __restrict__ slot_mapping, int H, int G, int Dv,
+    int maps, int rot, int bs, float eps, int by_map) {
+  using V8 = typename Vec<T>::v8;
+  constexpr int D = LPU * 8, UPB = 256 / LPU;
+  const long t = blockIdx.x;
+  const int tid = threadIdx.x, sub = tid % LPU, d0 = sub * 8;
+  const T* row = qkv + t * qkv_stride;
+  const int half = rot / 2, hl = half / 8;          // partner lane distance
+  const float* cs = rot > 0 ? cos_sin + positions[t] * (long)rot : nullptr;
+  const long slot = slot_mapping[t];
+  const int nq = H * maps, nk = G * maps, total = nq + nk;
+  for (int u0 = 0; u0 < total; u0 += UPB) {
+    const int u = u0 + tid / LPU;
+    const bool live = u < total;
+    const int uc = live ? u : total - 1;
+    const bool is_q = uc < nq;
+    const V8 v = ld16<V8>(row + (long)uc * D + d0);
+    const float* w = (is_q ? q_w : k_w) + d0;
+    float x[8], ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { x[i] = (float)v[i]; ss += x[i] * x[i]; }
+#pragma unroll
+    for (int o = LPU / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+    const float rs = 1.f / sqrtf(ss / (float)D + eps);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] *= rs * w[i];
+    if (rot > 0) {                                   // uniform
+      const bool lowh = d0 < half, turn = d0 < rot;
+      const int partner = (tid & 63) + (lowh ? hl : -hl);
+      const float* cp = cs + (lowh ? d0 : d0 - half);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float o = __shfl(x[i], partner & 63, 64);
+        if (turn) {
+          const float co = cp[i], si = cp[half + i];
+          x[i] = lowh ? x[i] * co - o * si : x[i] * co + o * si;
+        }
+      }
+    }
+    if (!live) continue;
+    T* dst;
+    if (is_q) {
+      int uo = u;
+      if (by_map) {
+        const int R = H / G, h = u / maps, mp = u % maps;
+        uo = ((h / R) * maps + mp) * R + h % R;
+      }
+      dst = qn + (t * nq + uo) * (long)D;
+    } else {
+      if (slot < 0) continue;
+      const int uk = u - nq;
+      const int g = uk / maps, mp = uk % maps;
+      dst = by_map ? k_cache + (((slot / bs) * nk + uk) * (long)bs + slot % bs) * (long)D
+                   : k_cache + (((slot / bs) * G + g) * (long)bs + slot % bs) * (long)(maps * D) + (long)mp * D;
+    }
+    V8 o8;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o8[i] = (T)x[i];
+    st16<V8>(dst + d0, o8);
+  }
+  if (slot >= 0) {
+    const T* vsrc = row + (long)total * D;
+    T* vdst = v_cache + (slot / bs) * (long)G * Dv * bs + slot % bs;      // [blocks, G, Dv, bs]
+    for (int e = tid; e < G * Dv; e += 256) vdst[(long)e * bs] = vsrc[e];
+  }
+}
+
 VDA_EXPORT int vda_qk_norm_rope_cache(void* qn, const void* qkv, long qkv_stride, const float* q_w, const float* k_w,
                                       const float* cos_sin, const long* positions, void* k_cache, void* v_cache,
                                       const long* slot_mapping, int T, int H, int G, int D, int Dv, int maps, int rot,
                                       int bs, float eps, int by_map, int dtype, hipStream_t st) {
   if (T <= 0) return 0;
   if (rot < 0 || rot > D || (rot & 1) || maps < 1 || (rot > 0 && !cos_sin)) return -1;
+  const bool vec = (D == 32 || D == 64 || D == 128 || D == 256) && (rot / 2) % 8 == 0 && qkv_stride % 8 == 0 &&
+                   ((uintptr_t)qkv % 32 == 0) && ((uintptr_t)qn % 32 == 0) && ((uintptr_t)k_cache % 32 == 0);
+  if (vec) {
+#define LV2(TT, LL) hipLaunchKernelGGL((qk_norm_rope_cache_vec_kernel<TT, LL>), dim3(T), dim3(256), 0, st, (TT*)qn,    \
+                                       (const TT*)qkv, qkv_stride, q_w, k_w, cos_sin, positions, (TT*)k_cache,          \
+                                       (TT*)v_cache, slot_mapping, H, G, Dv, maps, rot, bs, eps, by_map)
+#define LV(TT) do { if (D == 32) LV2(TT, 4); else if (D == 64) LV2(TT, 8); else if (D == 128) LV2(TT, 16); else LV2(TT, 32); } while (0)
+    if (dtype == VDA_BF16) LV(bf16_t);
+    else if (dtype == VDA_F16) LV(f16_t);
+    else if (dtype == VDA_F32) LV(float);
+    else return -3;
+#undef LV
+#undef LV2
+    VDA_CHECK_LAUNCH();
+    return 0;
+  }
 #define L(TT) hipLaunchKernelGGL((qk_norm_rope_cache_kernel<TT>), dim3(T), dim3(256), 0, st, (TT*)qn, (const TT*)qkv,  \
                                  qkv_stride, q_w, k_w, cos_sin, positions, (TT*)k_cache, (TT*)v_cache, slot_mapping,  \
                                  H, G, D, Dv, maps, rot, bs, eps, by_map)

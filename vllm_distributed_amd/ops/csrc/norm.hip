@@ -420,33 +420,74 @@ VDA_EXPORT int vda_residual_layer_norm(float* x, const void* y, long y_stride, c
 }
 
 // Dot products that a design wants in fp32 although the activations are 16-bit: out[t, r] = bias[r] + x[t, :] . w[r, :]
-// with fp32 weights (router logits, one-number gates).  One workgroup per token, a wave per output row in turn.
-template <typename T>
+// with fp32 weights (router logits, one-number gates).  A wave takes 8 tokens: per 512-column step it holds 8 weight
+// rows x 8 columns per lane in registers and streams the 8 tokens' values past them (16-byte loads), so weights come
+// from cache once per 8 tokens and every activation row is read once per group of 8 output rows; the 64 partial sums
+// are reduced over the lanes at the end.  Widths that are not a multiple of 8 take one value per lane and step.
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void fp32_rows_dot_kernel(float* __restrict__ out, const T* __restrict__ x,
                                                             long x_stride, const float* __restrict__ w,
-                                                            const float* __restrict__ bias, int R, int W) {
-  const long t = blockIdx.x;
+                                                            const float* __restrict__ bias, int T_, int R, int W) {
+  using V8 = typename Vec<T>::v8;
+  constexpr int TT = 8, RR = 8, CL = VEC ? 8 : 1;       // tokens and rows per pass, columns per lane and step
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const T* xr = x + t * x_stride;
-  for (int r = wave; r < R; r += 4) {
-    const float* wr = w + (long)r * W;
-    float a = 0.f;
-    for (int c = lane; c < W; c += 64) a += (float)xr[c] * wr[c];
-    a = wave_sum(a);
-    if (lane == 0) out[t * R + r] = a + (bias ? bias[r] : 0.f);
+  const long t0 = ((long)blockIdx.x * 4 + wave) * TT;
+  if (t0 >= T_) return;
+  for (int r0 = 0; r0 < R; r0 += RR) {
+    float acc[TT][RR];
+#pragma unroll
+    for (int a = 0; a < TT; ++a)
+#pragma unroll
+      for (int b = 0; b < RR; ++b) acc[a][b] = 0.f;
+    for (int c0 = lane * CL; c0 < W; c0 += 64 * CL) {
+      float wr[RR][CL];
+#pragma unroll
+      for (int b = 0; b < RR; ++b) {
+        const float* wp = w + (long)min(r0 + b, R - 1) * W + c0;
+#pragma unroll
+        for (int i = 0; i < CL; ++i) wr[b][i] = wp[i];
+      }
+#pragma unroll
+      for (int a = 0; a < TT; ++a) {
+        const T* xp = x + min(t0 + a, (long)T_ - 1) * x_stride + c0;
+        float xv[CL];
+        if (VEC) {
+          const V8 v = ld16<V8>(xp);
+#pragma unroll
+          for (int i = 0; i < CL; ++i) xv[i] = (float)v[i];
+        } else {
+          xv[0] = (float)xp[0];
+        }
+#pragma unroll
+        for (int b = 0; b < RR; ++b)
+#pragma unroll
+          for (int i = 0; i < CL; ++i) acc[a][b] += xv[i] * wr[b][i];
+      }
+    }
+#pragma unroll
+    for (int a = 0; a < TT; ++a)
+#pragma unroll
+      for (int b = 0; b < RR; ++b) {
+        const float v = wave_sum(acc[a][b]);
+        if (lane == 0 && t0 + a < T_ && r0 + b < R) out[(t0 + a) * R + r0 + b] = v + (bias ? bias[r0 + b] : 0.f);
+      }
   }
 }
 
 VDA_EXPORT int vda_fp32_rows_dot(float* out, const void* x, long x_stride, const float* w, const float* bias, int T,
                                  int R, int W, int dtype, hipStream_t st) {
   if (T <= 0 || R <= 0) return 0;
-#define L(TT) hipLaunchKernelGGL((fp32_rows_dot_kernel<TT>), dim3(T), dim3(256), 0, st, out, (const TT*)x, x_stride, \
-                                 w, bias, R, W)
+  const bool vec = W % 8 == 0 && x_stride % 8 == 0 && (uintptr_t)x % 32 == 0;
+  const dim3 grid((unsigned)((T + 31) / 32)), block(256);
+#define L2(TT, VV) hipLaunchKernelGGL((fp32_rows_dot_kernel<TT, VV>), grid, block, 0, st, out, (const TT*)x, x_stride, \
+                                      w, bias, T, R, W)
+#define L(TT) do { if (vec) L2(TT, true); else L2(TT, false); } while (0)
   if (dtype == VDA_BF16) L(bf16_t);
   else if (dtype == VDA_F16) L(f16_t);
   else if (dtype == VDA_F32) L(float);
   else return -3;
 #undef L
+#undef L2
   VDA_CHECK_LAUNCH();
   return 0;
 }
