@@ -310,6 +310,7 @@ VDA_EXPORT int vda_residual_norms(float* x, const void* y, long y_stride, const 
   else return -3;
 #undef L
 #undef L2
+#undef L3
   VDA_CHECK_LAUNCH();
   return 0;
 }
@@ -415,6 +416,7 @@ VDA_EXPORT int vda_residual_layer_norm(float* x, const void* y, long y_stride, c
   else return -3;
 #undef L
 #undef L2
+#undef L3
   VDA_CHECK_LAUNCH();
   return 0;
 }
@@ -424,12 +426,12 @@ VDA_EXPORT int vda_residual_layer_norm(float* x, const void* y, long y_stride, c
 // rows x 8 columns per lane in registers and streams the 8 tokens' values past them (16-byte loads), so weights come
 // from cache once per 8 tokens and every activation row is read once per group of 8 output rows; the 64 partial sums
 // are reduced over the lanes at the end.  Widths that are not a multiple of 8 take one value per lane and step.
-template <typename T, bool VEC>
+template <typename T, bool VEC, int TT>
 __global__ __launch_bounds__(256) void fp32_rows_dot_kernel(float* __restrict__ out, const T* __restrict__ x,
                                                             long x_stride, const float* __restrict__ w,
                                                             const float* __restrict__ bias, int T_, int R, int W) {
   using V8 = typename Vec<T>::v8;
-  constexpr int TT = 8, RR = 8, CL = VEC ? 8 : 1;       // tokens and rows per pass, columns per lane and step
+  constexpr int RR = 8, CL = VEC ? 8 : 1;       // rows per pass, columns per lane and step (TT: tokens per wave)
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const long t0 = ((long)blockIdx.x * 4 + wave) * TT;
   if (t0 >= T_) return;
@@ -478,9 +480,11 @@ VDA_EXPORT int vda_fp32_rows_dot(float* out, const void* x, long x_stride, const
                                  int R, int W, int dtype, hipStream_t st) {
   if (T <= 0 || R <= 0) return 0;
   const bool vec = W % 8 == 0 && x_stride % 8 == 0 && (uintptr_t)x % 32 == 0;
-  const dim3 grid((unsigned)((T + 31) / 32)), block(256);
-#define L2(TT, VV) hipLaunchKernelGGL((fp32_rows_dot_kernel<TT, VV>), grid, block, 0, st, out, (const TT*)x, x_stride, \
-                                      w, bias, T, R, W)
+  const bool many = T >= 4096;          // few tokens (decoding): one per wave, for the launch to spread over the chip
+  const dim3 grid((unsigned)(many ? (T + 31) / 32 : (T + 3) / 4)), block(256);
+#define L3(TT, VV, NT) hipLaunchKernelGGL((fp32_rows_dot_kernel<TT, VV, NT>), grid, block, 0, st, out, (const TT*)x,   \
+                                          x_stride, w, bias, T, R, W)
+#define L2(TT, VV) do { if (many) L3(TT, VV, 8); else L3(TT, VV, 1); } while (0)
 #define L(TT) do { if (vec) L2(TT, true); else L2(TT, false); } while (0)
   if (dtype == VDA_BF16) L(bf16_t);
   else if (dtype == VDA_F16) L(f16_t);
@@ -488,6 +492,7 @@ VDA_EXPORT int vda_fp32_rows_dot(float* out, const void* x, long x_stride, const
   else return -3;
 #undef L
 #undef L2
+#undef L3
   VDA_CHECK_LAUNCH();
   return 0;
 }
