@@ -182,7 +182,7 @@ def test_scaled_frequencies_against_the_oracle():
 
 # (heads, kv heads, D, Dv, maps, window, chunk, sink, rotated dims, gate)
 ATTN_SIZES = [(4, 2, 12, 20, 1, 9, 0, True, 8, False), (2, 1, 8, 12, 2, 0, 11, False, 4, True),
-              (6, 2, 64, 64, 1, 40, 0, True, 32, False), (4, 2, 32, 64, 2, 0, 32, False, 8, True),
+              (6, 3, 64, 64, 1, 37, 0, True, 16, False), (6, 2, 16, 40, 2, 0, 24, False, 6, True),
               (3, 3, 5, 7, 1, 0, 0, True, 0, False), (1, 1, 4, 2, 2, 1, 0, False, 4, False),
               (8, 1, 16, 16, 1, 33, 16, False, 16, True), (2, 2, 6, 70, 2, 0, 1, True, 2, False),
               (16, 2, 128, 128, 2, 0, 64, False, 64, True), (4, 4, 64, 64, 2, 24, 16, False, 16, False),
@@ -346,7 +346,7 @@ def test_short_convolution_in_ragged_portions(dev, taps):
 
 
 @pytest.mark.parametrize("dev,dt", OP_CASES)
-@pytest.mark.parametrize("Wd,ff,E,top,T", [(24, 10, 5, 2, 9), (33, 7, 3, 3, 4), (48, 96, 8, 4, 70), (256, 128, 8, 2, 150),
+@pytest.mark.parametrize("Wd,ff,E,top,T", [(24, 10, 5, 2, 9), (33, 7, 3, 3, 4), (48, 80, 6, 3, 70), (256, 128, 8, 2, 150),
                                            (128, 64, 4, 1, 3)])
 def test_experts_without_a_gate_half(dev, dt, Wd, ff, E, top, T):
     """Routing (largest logits with a bias, softmax over the chosen ones) and the experts' sum; the last sizes are ones
