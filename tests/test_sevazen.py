@@ -141,11 +141,14 @@ def test_residual_with_output_layer_norm(dev, dt, W_):
 
 
 @pytest.mark.parametrize("dev,dt", OP_CASES)
-def test_fp32_dot_products_of_16_bit_rows(dev, dt):
-    x, w, b = torch.randn(9, 77).to(dt), torch.randn(5, 77), torch.randn(5)
-    got = ops.fp32_rows_dot(x.to(dev)[:, :70], w[:, :70].contiguous().to(dev), b.to(dev))
+@pytest.mark.parametrize("T,W_,R", [(9, 70, 5), (33, 128, 9), (4100, 70, 3), (4099, 640, 17)])
+def test_fp32_dot_products_of_16_bit_rows(dev, dt, T, W_, R):
+    """Few rows (one token per wave) and many (eight per wave, sums exchanged between lanes); widths with and without
+    16-byte steps; more output rows than one pass holds."""
+    x, w, b = torch.randn(T, W_ + 8).to(dt), torch.randn(R, W_), torch.randn(R)
+    got = ops.fp32_rows_dot(x.to(dev)[:, :W_], w.to(dev), b.to(dev))
     assert got.dtype == torch.float32
-    torch.testing.assert_close(got.cpu(), x[:, :70].float() @ w[:, :70].T + b, atol=1e-4, rtol=1e-5)
+    torch.testing.assert_close(got.cpu(), x[:, :W_].float() @ w.T + b, atol=2e-4, rtol=1e-5)
 
 
 def rot_table(rot, kind, n, dev):

@@ -466,13 +466,30 @@ __global__ __launch_bounds__(256) void fp32_rows_dot_kernel(float* __restrict__ 
           for (int i = 0; i < CL; ++i) acc[a][b] += xv[i] * wr[b][i];
       }
     }
+    if (TT * RR == 64) {
+      // 64 sums over 64 lanes in 63 exchanges instead of 64 x 6: at every step a lane keeps one half of its values and
+      // hands the other half to its partner; in the end lane L holds the total of value L = (token L / 8, row L % 8)
+      float* f = &acc[0][0];
 #pragma unroll
-    for (int a = 0; a < TT; ++a)
+      for (int o = 32; o >= 1; o >>= 1) {
+        const bool up = lane & o;
 #pragma unroll
-      for (int b = 0; b < RR; ++b) {
-        const float v = wave_sum(acc[a][b]);
-        if (lane == 0 && t0 + a < T_ && r0 + b < R) out[(t0 + a) * R + r0 + b] = v + (bias ? bias[r0 + b] : 0.f);
+        for (int i = 0; i < o; ++i) {
+          const float keep = up ? f[i + o] : f[i], give = up ? f[i] : f[i + o];
+          f[i] = keep + __shfl_xor(give, o, 64);
+        }
       }
+      const int a = lane / RR, b = lane % RR;
+      if (t0 + a < T_ && r0 + b < R) out[(t0 + a) * R + r0 + b] = f[0] + (bias ? bias[r0 + b] : 0.f);
+    } else {
+#pragma unroll
+      for (int a = 0; a < TT; ++a)
+#pragma unroll
+        for (int b = 0; b < RR; ++b) {
+          const float v = wave_sum(acc[a][b]);
+          if (lane == 0 && t0 + a < T_ && r0 + b < R) out[(t0 + a) * R + r0 + b] = v + (bias ? bias[r0 + b] : 0.f);
+        }
+    }
   }
 }
 
