@@ -473,11 +473,12 @@ def test_unequal_requests_share_steps_and_reuse_pages_and_slots(tmp_path, dev, d
     check(cfg, W, prompts, got, dtype)
 
 
-def needle_model():
+def needle_model(window=40, chunk=64):
     """Token 0 is a 'needle': in the window layer and in the chunk layer one head's queries look for it and it takes
     nearly all the weight while the mask lets it through, so the logits move by O(1) where it enters or leaves."""
-    layers = [O.window_layer(heads=2, kv_heads=1, dim=8, vdim=8, window=40, conv=None, rot_dims=0, scale=1.0, mlp=None),
-              O.diff_layer(heads=2, kv_heads=1, dim=8, vdim=8, chunk=64, rot_dims=0, scale=1.0, diff=0.2, mlp=None)]
+    layers = [O.window_layer(heads=2, kv_heads=1, dim=8, vdim=8, window=window, conv=None, rot_dims=0, scale=1.0,
+                             mlp=None),
+              O.diff_layer(heads=2, kv_heads=1, dim=8, vdim=8, chunk=chunk, rot_dims=0, scale=1.0, diff=0.2, mlp=None)]
     cfg = O.make_config(layers, vocab=64, width=32)
     W = {k: v.float() for k, v in O.make_weights(cfg, 11).items()}
     emb = 0.2 * W["embed"]
@@ -523,6 +524,25 @@ def test_far_key_and_edges_that_matter(tmp_path, dev, dtype):
         cfg2 = O.make_config(ls, vocab=64, width=32)
         full = O.forward(cfg, W, prompts[rid])
         assert O.logit_error(O.forward(cfg2, W, prompts[rid])[pos], full[pos]) > 0.05, (which, rid)
+
+
+@pytest.mark.parametrize("dev,dtype", CASES)
+def test_far_key_among_hundreds(tmp_path, dev, dtype):
+    """Wide masks (a window of 300, chunks of 320): the one key that matters sits hundreds of tokens and many pages
+    back, leaves the window while single tokens are decoded and the chunk inside a prompt portion."""
+    layers, cfg, W = needle_model(window=300, chunk=320)
+    folder = O.save_checkpoint(str(tmp_path / "m"), cfg, W)
+    V = cfg["vocab"]
+    body = [t % (V - 1) + 1 for t in tokens(400, V, 14)]
+    p = body[:5] + [0] + body[5:345]                       # needle at 5: in the window up to 304, in the chunk up to 319
+    sched = [[("deep", 290)]] + [[("deep", 1)]] * 22 + [[("deep", 2)], [("deep", 3)], [("deep", 29)]]
+    got = run_schedule(folder, dtype, dev, {"deep": p}, sched, 384)
+    check(cfg, W, {"deep": p}, got, dtype)
+    full = O.forward(cfg, W, p)
+    for which, size, pos in ((0, 299, 304), (1, 319, 319)):
+        ls = [dict(l, mixer=dict(l["mixer"])) for l in layers]
+        ls[which]["mixer"]["mask"] = {"size": size}
+        assert O.logit_error(O.forward(O.make_config(ls, vocab=64, width=32), W, p)[pos], full[pos]) > 0.05, which
 
 
 @pytest.mark.parametrize("dev", DEVICES)
