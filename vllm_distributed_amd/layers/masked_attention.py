@@ -2,7 +2,8 @@
 on the projections, several score maps per head, window / chunk masks, sinks and an output gate.
 
     q, k, v = W x + b                                   (optional biases; grouped query heads; key width D, value width Dv)
-    q, k, v <- causal convolution over time, per channel (``conv_taps`` > 1; no bias, no activation)
+    q, k, v <- causal convolution over time, per channel (``conv_taps`` >= 1; no bias, no activation; one tap is a
+               weight per channel)
     q, k    <- q / rms(q) * q_norm, k / rms(k) * k_norm  per head and map (weights of size D shared by all heads)
     q, k    <- first ``rot_dims`` values of each map rotated, value i paired with i + rot_dims / 2 (fp32 angles)
     score   = scale * q . k;   key j visible to query i: j <= i, i - j < window, j // chunk == i // chunk
@@ -17,7 +18,11 @@ keys that a window or chunk hides stay in their pages, the kernels never load th
 slot per request for the last ``conv_taps - 1`` projected rows (the slots of the recurrent mixers).  A stack that runs
 one set of weights at several depths gives every use a cache and state of its own (``users``).
 Cache layout: K [blocks, G, block, maps * D] (normed and rotated), V [blocks, G, Dv, block].
-Kernels: ops/csrc/masked_attention.hip, ops/csrc/mamba.hip (the convolution shared with the state-space mixers).
+With 16-bit activations and keys and values of one width that the matrix-core paged attention kernels are built for,
+those kernels run (ops/csrc/attention.hip with the window, chunk and sink as options); every score map is then a key
+head of its own in the cache, K [blocks, G * maps, block, D] in the same memory, and an epilogue kernel combines the maps.
+Kernels: ops/csrc/masked_attention.hip, ops/csrc/attention.hip, ops/csrc/mamba.hip (the convolution shared with the
+state-space mixers).
 """
 from __future__ import annotations
 
