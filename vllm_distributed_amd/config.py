@@ -173,6 +173,9 @@ def load_hf_config(model: str, overrides: Optional[dict] = None) -> HFConfig:
     if d.get("architecture") == "Sevazen":         # a layer list of attention variants; layers may share weights
         from .models.sevazen import normalise_config as sevazen_config
         d = sevazen_config(d, model if os.path.isdir(model) else None)
+    if d.get("architecture") == "Lefolorn":        # a layer list of three attention variants with parallel sub-layers
+        from .models.lefolorn import normalise_config as lefolorn_config
+        d = lefolorn_config(d, model if os.path.isdir(model) else None)
     if d.get("model_type") in ("exaone", "telechat", "qwen", "chatglm"):
         from .models.renamed_decoders import normalise_config
         d = normalise_config(d)

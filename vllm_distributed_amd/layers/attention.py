@@ -507,9 +507,10 @@ class MLAAttention(nn.Module):
                           md.query_start_loc[:S + 1], self.scale, md.max_query_len, nsplit, self._kv_scale_float)
         return out
 
-    def forward_cached(self, q: torch.Tensor) -> torch.Tensor:
+    def forward_cached(self, q: torch.Tensor, sink: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Attention over rows the caller has already written to the cache for this step's tokens.
-        q [T, H, dk]; returns [T, H, kv_lora_rank]."""
+        q [T, H, dk]; returns [T, H, kv_lora_rank].  ``sink`` fp32 [H]: exp(sink[h]) joins head h's softmax
+        denominator, with no key and no value."""
         md: Optional[AttentionMetadata] = get_forward_context().attn_metadata
         T = q.shape[0]
         if md is None or self.k_cache is None:
@@ -523,7 +524,7 @@ class MLAAttention(nn.Module):
             # the batch's leading decode sequences (few query tokens: the keys split over waves and workgroups), then
             # its prompts and portions (key steps staged in LDS for several tokens), as the other attention layers do
             nd, ndt, n_pre = md.num_decode_seqs, md.num_decode_tokens, md.num_prefill_seqs
-            kw = dict(kv_scale=self._kv_scale_float, window=self.sliding_window)
+            kw = dict(kv_scale=self._kv_scale_float, window=self.sliding_window, sink=sink)
             if nd > 0:
                 keys = min(self.max_model_len, self.sliding_window + 32) if self.sliding_window else self.max_model_len
                 nsplit = ops.decode_num_splits(nd * max(self.num_heads // 16, 1), 1, keys)
@@ -538,7 +539,7 @@ class MLAAttention(nn.Module):
             return out
         out = ops.latent_window_attention(q[:n], self.k_cache, md.block_table[:S], md.seq_lens[:S],
                                           md.query_start_loc[:S + 1], self.scale, self.sliding_window, self.dv,
-                                          md.max_query_len)
+                                          md.max_query_len, sink)
         if n < T:
             out = torch.cat([out, out.new_zeros((T - n, self.num_heads, self.dv))], dim=0)
         return out

@@ -1,10 +1,12 @@
 """Latent attention over a sliding window: keys and values are up-projections of one low-rank latent per token,
 plus a rotated key part that all heads share; only the latent and that part are cached.
 
-    q = W_q x                      per head [D plain | P rotated]
+    q = W_q x                      per head [D plain | P rotated]; with ``q_rank``: q = W_uq (W_dq x / rms * q_norm), the
+                                   queries through a normed latent of their own
     [c_raw | k_rot] = W_dkv x      c = c_raw / rms(c_raw) * c_norm  (R values);  k_rot: P values, rotated, no norm
     k_h = W_uk_h c,  v_h = W_uv_h c
     score(i, j, h) = scale * (q_plain . k_h + q_rot . k_rot),   j <= i and i - j < window,   softmax over j
+                                   (``sink``: a learned number per head whose exponential joins the denominator)
     out = W_o [sum_j p v_h]_h
 
 The rotation turns the pairs (2i, 2i + 1), i < rot_dims / 2, of the P rotated values by position * base^(-2i / rot_dims)
@@ -28,7 +30,7 @@ from ..forward_context import get_forward_context
 from ..parallel.state import get_tensor_model_parallel_world_size
 from .attention import MLAAttention
 from .hyper_connections import _fp32_param
-from .linear import ReplicatedLinear, RowParallelLinear
+from .linear import MergedColumnParallelLinear, ReplicatedLinear, RowParallelLinear
 
 _TABLES: dict = {}
 
@@ -51,7 +53,7 @@ def interleaved_cos_sin(max_len: int, dims: int, base: float, device) -> torch.T
 class WindowedLatentAttention(nn.Module):
     def __init__(self, hidden_size: int, num_heads: int, head_dim: int, rot_dim: int, v_head_dim: int, kv_rank: int,
                  scale: float, window: Optional[int], rot_base: Optional[float], rot_dims: int, eps: float,
-                 passes: int = 1, quant_config=None, prefix: str = ""):
+                 passes: int = 1, quant_config=None, prefix: str = "", q_rank: int = 0, sink: bool = False):
         super().__init__()
         if get_tensor_model_parallel_world_size() > 1:
             raise NotImplementedError("windowed latent attention runs with tensor_parallel_size=1")
@@ -61,10 +63,20 @@ class WindowedLatentAttention(nn.Module):
         self.rot_dims = int(rot_dims) if rot_base else 0
         if self.rot_dims > P or self.rot_dims % 2:
             raise ValueError(f"{prefix}: {self.rot_dims} rotated dimensions do not fit an even part of {P}")
-        self.q_proj = ReplicatedLinear(hidden_size, H * (D + P), bias=False, quant_config=quant_config,
-                                       prefix=f"{prefix}.q_proj")
-        self.dkv_proj = ReplicatedLinear(hidden_size, R + P, bias=False, quant_config=quant_config,
-                                         prefix=f"{prefix}.dkv_proj")
+        self.q_rank = int(q_rank or 0)
+        if self.q_rank:
+            # one GEMM for both down-projections: [query latent | key / value latent + rotated key part]
+            self.down_proj = MergedColumnParallelLinear(hidden_size, [self.q_rank, R + P], bias=False,
+                                                        quant_config=quant_config, prefix=f"{prefix}.down_proj")
+            self.q_norm = _fp32_param((self.q_rank,))
+            self.uq_proj = ReplicatedLinear(self.q_rank, H * (D + P), bias=False, quant_config=quant_config,
+                                            prefix=f"{prefix}.uq_proj")
+        else:
+            self.q_proj = ReplicatedLinear(hidden_size, H * (D + P), bias=False, quant_config=quant_config,
+                                           prefix=f"{prefix}.q_proj")
+            self.dkv_proj = ReplicatedLinear(hidden_size, R + P, bias=False, quant_config=quant_config,
+                                             prefix=f"{prefix}.dkv_proj")
+        self.sink = _fp32_param((H,), 0.0) if sink else None
         self.uk_proj = ReplicatedLinear(R, H * D, bias=False, prefix=f"{prefix}.uk_proj")
         self.uv_proj = ReplicatedLinear(R, H * Dv, bias=False, prefix=f"{prefix}.uv_proj")
         self.o_proj = RowParallelLinear(H * Dv, hidden_size, bias=False, quant_config=quant_config,
@@ -103,8 +115,13 @@ class WindowedLatentAttention(nn.Module):
         attn = self.attn[pass_index]
         H, D, P, Dv, R = self.num_heads, self.head_dim, self.rot_dim, self.v_head_dim, self.kv_rank
         T = x.shape[0]
-        q = self.q_proj(x)
-        down = self.dkv_proj(x)
+        if self.q_rank:
+            both = self.down_proj(x)
+            q = self.uq_proj(ops.group_rms_norm(both[:, : self.q_rank], self.q_norm, self.eps, 1))
+            down = both[:, self.q_rank:]
+        else:
+            q = self.q_proj(x)
+            down = self.dkv_proj(x)
         w_uk, w_uv_t = self._folded_weights()
         qf = torch.empty((T, H, R + P), dtype=q.dtype, device=q.device)
         q3 = q.view(T, H, D + P)
@@ -120,6 +137,6 @@ class WindowedLatentAttention(nn.Module):
             ops.latent_norm_rope_cache(q[:n], down[:n], self.c_norm, self._tables(q.device), positions[:n], qf[:n],
                                        attn.k_cache, md.slot_mapping[:n], H, D, P, R, self.rot_dims, self.eps,
                                        attn.v_cache if self.use_mfma else None)
-            o_lat = attn.forward_cached(qf)
+            o_lat = attn.forward_cached(qf, self.sink)
         o = torch.bmm(o_lat.transpose(0, 1), w_uv_t).transpose(0, 1)
         return self.o_proj(o.reshape(T, H * Dv))

@@ -5,9 +5,17 @@ on the projections, several score maps per head, window / chunk masks, sinks and
     q, k, v <- causal convolution over time, per channel (``conv_taps`` >= 1; no bias, no activation; one tap is a
                weight per channel)
     q, k    <- q / rms(q) * q_norm, k / rms(k) * k_norm  per head and map (weights of size D shared by all heads)
-    q, k    <- first ``rot_dims`` values of each map rotated, value i paired with i + rot_dims / 2 (fp32 angles)
-    score   = scale * q . k;   key j visible to query i: j <= i, i - j < window, j // chunk == i // chunk
-    softmax over the visible keys; with ``sink`` the denominator also holds exp(sink[h])
+    q, k    <- first ``rot_dims`` values of each map rotated, value i paired with i + rot_dims / 2 (``rot_pairing``
+               "halves") or value 2i with 2i + 1 ("neighbours"), fp32 angles
+    q       <- q * (1 + coef * ln(floor((p + 1) / every) + 1)) at position p (``q_temp`` = (coef, every))
+    v       <- (1 - lam) v + lam v_first (``v_mix``): v_first are the values that the first such layer of the stack
+               made of the same token; the layers of one forward pass hand them on through a dictionary
+    score   = scale * q . k;  score <- cap * tanh(score / cap) (``softcap``);  score += rel[bucket(i - j), h]
+               (``dist_bias`` = (rows, far): distances below rows / 2 have a row each, the others share the rest in
+               logarithmic steps up to ``far``)
+    key j visible to query i: j <= i, i - j < window, j // chunk == i // chunk
+    softmax over the visible keys; with ``sink`` the denominator also holds exp(sink[h]) (a learned number per head),
+               with ``sink_fixed`` = s it holds exp(s) (s = 0: one more 1)
     maps == 2 (differential attention): a head's query / key rows hold two maps side by side, each an attention over
                the same values;  o = a1 - lam * a2,  lam = exp(lq1 . lk1) - exp(lq2 . lk2) + diff,
                then o / rms(o) * (1 - diff) over the head's Dv values
@@ -40,6 +48,21 @@ from ..sched.kv_cache_interface import FullAttentionSpec, KVCacheSpec
 from .hyper_connections import _fp32_param
 from .linear import MergedColumnParallelLinear, RowParallelLinear, set_weight_attrs
 from .rotary import half_split_cos_sin
+
+
+def log_bucket_rows(rows: int, far: int) -> torch.Tensor:
+    """Row of a distance table for every distance 0 .. far: n itself below rows / 2, then
+    min(rows - 1, rows / 2 + floor(ln(n / (rows / 2)) / ln(far / (rows / 2)) * (rows - rows / 2)));
+    ``far`` and everything beyond share the last row.  int64 [far + 1]."""
+    import math
+    half = rows // 2
+    out = []
+    for n in range(int(far) + 1):
+        if n < half or half == 0:
+            out.append(min(n, rows - 1))
+        else:
+            out.append(min(rows - 1, half + int(math.floor(math.log(n / half) / math.log(far / half) * (rows - half)))))
+    return torch.tensor(out, dtype=torch.int64)
 
 
 class PagedKV(nn.Module):
@@ -80,7 +103,8 @@ class MaskedSoftmaxAttention(nn.Module):
                  scale: float, eps: float, *, bias: bool = False, conv_taps: int = 0, window: int = 0, chunk: int = 0,
                  sink: bool = False, maps: int = 1, diff: float = 0.0, gate: bool = False, rot_dims: int = 0,
                  rot_base: float = 10000.0, rot_scaling: Optional[dict] = None, users: int = 1, quant_config=None,
-                 prefix: str = ""):
+                 prefix: str = "", rot_pairing: str = "halves", q_temp: Optional[tuple] = None, softcap: float = 0.0,
+                 dist_bias: Optional[tuple] = None, sink_fixed: Optional[float] = None, v_mix: bool = False):
         super().__init__()
         if get_tensor_model_parallel_world_size() > 1:
             raise NotImplementedError("this attention layer runs with tensor_parallel_size=1")
@@ -96,6 +120,15 @@ class MaskedSoftmaxAttention(nn.Module):
         self.window, self.chunk, self.maps, self.diff = int(window or 0), int(chunk or 0), int(maps), float(diff)
         self.taps = int(conv_taps or 0)
         self.rot_dims, self.rot_base, self.rot_scaling = int(rot_dims), float(rot_base), rot_scaling
+        if rot_pairing not in ("halves", "neighbours") or (rot_pairing == "neighbours" and rot_scaling):
+            raise ValueError(f"{prefix}: rotation pairing {rot_pairing!r} (with frequency scaling: halves only)")
+        if sink and sink_fixed is not None:
+            raise ValueError(f"{prefix}: a learned sink and a fixed one exclude each other")
+        self.rot_pairing = rot_pairing
+        self.q_temp = (float(q_temp[0]), int(q_temp[1])) if q_temp else None
+        if self.q_temp and self.q_temp[1] < 1:
+            raise ValueError(f"{prefix}: the query temperature grows every {self.q_temp[1]} positions")
+        self.softcap = float(softcap or 0.0)
         self.layer_name = prefix
         nq, nk, nv = H * maps * D, G * maps * D, G * Dv
         self.qkv_width = nq + nk + nv
@@ -108,7 +141,20 @@ class MaskedSoftmaxAttention(nn.Module):
                                         prefix=f"{prefix}.o_proj")
         self.q_norm = _fp32_param((D,))
         self.k_norm = _fp32_param((D,))
-        self.sink = _fp32_param((H,), 0.0) if sink else None
+        if sink_fixed is not None:
+            self.register_buffer("sink", torch.full((H,), float(sink_fixed), dtype=torch.float32), persistent=False)
+        else:
+            self.sink = _fp32_param((H,), 0.0) if sink else None
+        # learned bias per (distance bucket, head); the kernels read one row per distance, made once after loading
+        self.dist_far = 0
+        if dist_bias:
+            rows, self.dist_far = int(dist_bias[0]), int(dist_bias[1])
+            if rows < 2 or self.dist_far <= rows // 2:
+                raise ValueError(f"{prefix}: {rows} distance buckets up to {self.dist_far}")
+            self.rel = _fp32_param((rows, H), 0.0)
+            self.register_buffer("_bucket", log_bucket_rows(rows, self.dist_far), persistent=False)
+        self._dist_table: Optional[torch.Tensor] = None
+        self.vmix = _fp32_param((1,), 0.0) if v_mix else None
         if maps == 2:
             self.lq1, self.lk1 = _fp32_param((D,), 0.0), _fp32_param((D,), 0.0)
             self.lq2, self.lk2 = _fp32_param((D,), 0.0), _fp32_param((D,), 0.0)
@@ -132,9 +178,9 @@ class MaskedSoftmaxAttention(nn.Module):
         cfg = get_current_vllm_config()
         # 16-bit activations and head widths the matrix-core paged attention kernels are built for: those kernels (every
         # score map a key head of its own in the cache); anything else, fp32 included: the kernel for any sizes
-        self.use_mfma = ops.masked_attention_mfma_ok(H, G, D, Dv, maps, bool(sink), cfg.model_config.dtype,
+        self.use_mfma = ops.masked_attention_mfma_ok(H, G, D, Dv, maps, self.sink is not None, cfg.model_config.dtype,
                                                      cfg.device_config.device != "cpu") \
-            and cfg.cache_config.cache_dtype == "auto"
+            and cfg.cache_config.cache_dtype == "auto" and not self.dist_far
         self.max_len = int(cfg.model_config.max_model_len) + 1
         self._cos_sin: Optional[torch.Tensor] = None
 
@@ -142,8 +188,22 @@ class MaskedSoftmaxAttention(nn.Module):
         if self.rot_dims == 0:
             return None
         if self._cos_sin is None or self._cos_sin.device != device:
-            self._cos_sin = half_split_cos_sin(self.max_len, self.rot_dims, self.rot_base, self.rot_scaling, device)
+            if self.rot_pairing == "neighbours":
+                from .latent_attention import interleaved_cos_sin
+                self._cos_sin = interleaved_cos_sin(self.max_len, self.rot_dims, self.rot_base, device)
+            else:
+                self._cos_sin = half_split_cos_sin(self.max_len, self.rot_dims, self.rot_base, self.rot_scaling,
+                                                   device)
         return self._cos_sin
+
+    def _distances(self) -> Optional[torch.Tensor]:
+        """fp32 [far + 1, H]: the bias of every distance, the learned rows spread over their buckets (made once from
+        the loaded table)."""
+        if not self.dist_far:
+            return None
+        if self._dist_table is None or self._dist_table.device != self.rel.device:
+            self._dist_table = self.rel.data[self._bucket.to(self.rel.device)].contiguous()
+        return self._dist_table
 
     def _lambda(self) -> Optional[torch.Tensor]:
         """The weight of the second map, one fp32 value on the device (made once from the loaded vectors)."""
@@ -154,7 +214,10 @@ class MaskedSoftmaxAttention(nn.Module):
                          + self.diff).reshape(1).contiguous()
         return self._lam
 
-    def forward(self, x: torch.Tensor, positions: torch.Tensor, user: int = 0) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, positions: torch.Tensor, user: int = 0,
+                lent: Optional[dict] = None) -> torch.Tensor:
+        """``lent``: a dictionary that lives for one forward pass of the stack; the first layer with ``v_mix`` puts its
+        values there ("v_first") and the later ones mix them into their own."""
         md = get_forward_context().attn_metadata
         H, G, D, Dv, maps = self.num_heads, self.num_kv_heads, self.head_dim, self.v_head_dim, self.maps
         kv = self.caches[user]
@@ -177,10 +240,18 @@ class MaskedSoftmaxAttention(nn.Module):
         elif self.taps == 1:
             qkv = (p[:n, :W].float() * self.conv_weight.float().view(1, -1)).to(p.dtype)
         g_rows = gate[:n] if gate is not None else None
+        extras = dict(pairing=self.rot_pairing, q_temp=self.q_temp)
+        if self.vmix is not None:
+            if lent is None:
+                raise ValueError(f"{self.layer_name}: value mixing needs the forward pass's dictionary")
+            if "v_first" in lent:
+                extras.update(v_first=lent["v_first"], v_lam=self.vmix)
+            else:
+                lent["v_first"] = qkv[:, (H + G) * maps * D: (H + G) * maps * D + G * Dv]
         if self.use_mfma:
             qn = ops.qk_norm_rope_cache(qkv, H, G, D, Dv, maps, self.q_norm, self.k_norm, self._table(p.device),
                                         positions[:n], self.rot_dims, self.eps, kv.k_cache, kv.v_cache,
-                                        md.slot_mapping[:n], by_map=True)
+                                        md.slot_mapping[:n], by_map=True, **extras)
             nd, ndt, n_pre, npt, pqsl = (md.num_decode_seqs, md.num_decode_tokens, md.num_prefill_seqs,
                                          md.num_prefill_tokens, md.prefill_query_start_loc)
             cols = max(md.max_decode_query_len, 1) * (H // G)
@@ -190,17 +261,19 @@ class MaskedSoftmaxAttention(nn.Module):
             out = ops.masked_softmax_attention_mfma(
                 qn, kv.k_cache, kv.v_cache, md.block_table, md.seq_lens, md.query_start_loc, pqsl, nd, ndt, n_pre, npt,
                 md.max_decode_query_len, md.decode_num_splits, md.max_query_len, self.scale, H, self.window,
-                self.chunk, self.sink, maps, self._lambda(), self.eps, 1.0 - self.diff, g_rows)
+                self.chunk, self.sink, maps, self._lambda(), self.eps, 1.0 - self.diff, g_rows,
+                softcap=self.softcap, dist_bias=self._distances())
             if n < T:
                 out = torch.cat([out, out.new_zeros((T - n, out.shape[1]))], dim=0)
             return self.o_proj(out)
         qn = ops.qk_norm_rope_cache(qkv, H, G, D, Dv, maps, self.q_norm, self.k_norm, self._table(p.device),
                                     positions[:n], self.rot_dims, self.eps, kv.k_cache, kv.v_cache,
-                                    md.slot_mapping[:n])
+                                    md.slot_mapping[:n], **extras)
         out = ops.masked_softmax_attention(qn, kv.k_cache, kv.v_cache, md.block_table[:S], lens, qsl, self.scale,
                                            self.window, self.chunk, self.sink, maps, self._lambda(), self.eps,
                                            1.0 - self.diff, gate[:n] if gate is not None else None,
-                                           md.max_query_len, p.dtype)
+                                           md.max_query_len, p.dtype, softcap=self.softcap,
+                                           dist_bias=self._distances())
         if n < T:
             out = torch.cat([out, out.new_zeros((T - n, out.shape[1]))], dim=0)
         return self.o_proj(out)

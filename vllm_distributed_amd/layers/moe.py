@@ -44,12 +44,14 @@ def determine_expert_map(ep_size: int, ep_rank: int, global_num_experts: int) ->
 
 
 def grouped_topk(scores: torch.Tensor, k: int, renormalize: bool, num_expert_group: int, topk_group: int,
-                 bias: Optional[torch.Tensor] = None):
-    """DeepSeek-style routing: keep the best ``topk_group`` groups of experts, then top-k inside."""
+                 bias: Optional[torch.Tensor] = None, group_score: Optional[str] = None, renorm_eps: float = 0.0):
+    """DeepSeek-style routing: keep the best ``topk_group`` groups of experts, then top-k inside.  A group scores the
+    sum of its two best members (``group_score`` "top2", the default with a bias) or its best one ("max")."""
     T, E = scores.shape
     sel = scores + bias.unsqueeze(0) if bias is not None else scores
     g = sel.view(T, num_expert_group, -1)
-    gscore = g.topk(min(2, g.shape[-1]), dim=-1)[0].sum(-1) if bias is not None else g.max(dim=-1).values
+    top2 = (bias is not None) if group_score is None else group_score == "top2"
+    gscore = g.topk(min(2, g.shape[-1]), dim=-1)[0].sum(-1) if top2 else g.max(dim=-1).values
     gidx = gscore.topk(topk_group, dim=-1, sorted=False)[1]
     gmask = torch.zeros_like(gscore).scatter_(1, gidx, 1.0)
     mask = gmask.unsqueeze(-1).expand(T, num_expert_group, E // num_expert_group).reshape(T, E)
@@ -57,7 +59,7 @@ def grouped_topk(scores: torch.Tensor, k: int, renormalize: bool, num_expert_gro
     ids = masked.topk(k, dim=-1, sorted=False)[1]
     w = scores.gather(1, ids)
     if renormalize:
-        w = w / w.sum(dim=-1, keepdim=True)
+        w = w / (w.sum(dim=-1, keepdim=True) + renorm_eps)
     return w.float(), ids.to(torch.int32)
 
 
@@ -89,8 +91,20 @@ class FusedMoE(nn.Module):
                  topk_group: Optional[int] = None, quant_config=None, prefix: str = "",
                  custom_routing_function: Optional[Callable] = None, scoring_func: str = "softmax",
                  e_score_correction_bias: Optional[torch.Tensor] = None, routed_scaling_factor: float = 1.0,
-                 activation: str = "silu", act_limit: float = 0.0, gated: bool = True):
+                 activation: str = "silu", act_limit: float = 0.0, gated: bool = True,
+                 group_score: Optional[str] = None, num_identity_experts: int = 0, renorm_eps: float = 0.0,
+                 add_identity: bool = True):
         super().__init__()
+        # group_score: "top2" / "max", what a group of experts scores in group-limited choice (None: top2 with a
+        # selection bias, max without).  num_identity_experts: the router's last outputs have no expert behind them,
+        # their "expert" returns its input; the router then has num_experts + num_identity_experts outputs.  The
+        # weights such choices won are kept per token in ``identity_weight`` (fp32 [T]) by every forward; with
+        # ``add_identity`` the layer adds identity_weight * x itself, without the caller does (inside a fused pass).
+        self.group_score, self.renorm_eps = group_score, float(renorm_eps)
+        self.num_identity, self.add_identity = int(num_identity_experts), bool(add_identity)
+        self.identity_weight: Optional[torch.Tensor] = None
+        if self.num_identity and not use_grouped_topk:
+            raise NotImplementedError(f"{prefix}: identity experts come with group-limited choice (one group at least)")
         # gated=False: experts of the form W2 act(W1 x), no second (up) half; their first weight loads as "w1"
         self.gated = bool(gated)
         if not self.gated and quant_config is not None and quant_config.get_quant_method(self, prefix) is not None:
@@ -211,6 +225,8 @@ class FusedMoE(nn.Module):
         if self.custom_routing_function is not None:
             w, ids = self.custom_routing_function(router_logits, k, self.renormalize)
             return w.float(), ids.to(torch.int32)
+        if self.use_grouped_topk and (self.num_identity or self.group_score is not None or self.renorm_eps):
+            return self._select_grouped(router_logits)
         if self.use_grouped_topk and self.scoring_func == "sigmoid" and self.e_score_correction_bias is not None:
             # one launch: scores, group scores, the groups that stay, the choice and its weights
             routed = ops.moe_grouped_sigmoid_topk(router_logits, self.e_score_correction_bias, k,
@@ -229,6 +245,29 @@ class FusedMoE(nn.Module):
                 w = w / w.sum(-1, keepdim=True)
             return w, ids.to(torch.int32)
         return ops.moe_topk_softmax(router_logits, k, self.renormalize)
+
+    def _select_grouped(self, router_logits: torch.Tensor):
+        """Group-limited choice with every option (scoring, group score, identity outputs, renormalisation constant):
+        one launch on the device, PyTorch ops elsewhere.  Identity winners come back as id -1 / weight 0; their
+        weights' sum per token lands in ``identity_weight``."""
+        k, E = self.top_k, self.global_num_experts
+        top2 = (self.e_score_correction_bias is not None) if self.group_score is None else self.group_score == "top2"
+        routed = ops.moe_grouped_topk(router_logits, self.e_score_correction_bias, k, self.num_expert_group,
+                                      self.topk_group, self.renormalize, self.scoring_func,
+                                      "top2" if top2 else "max", self.num_identity, self.renorm_eps)
+        if routed is not None:
+            w, ids, self.identity_weight = routed
+            return w, ids
+        scores = torch.softmax(router_logits.float(), -1) if self.scoring_func == "softmax" \
+            else torch.sigmoid(router_logits.float())
+        w, ids = grouped_topk(scores, k, self.renormalize, self.num_expert_group, self.topk_group,
+                              self.e_score_correction_bias, "top2" if top2 else "max", self.renorm_eps)
+        if self.num_identity:
+            ident = ids >= E
+            self.identity_weight = (w * ident).sum(-1)
+            w = w.masked_fill(ident, 0.0)
+            ids = ids.masked_fill(ident, -1)
+        return w, ids
 
     def _forward_ep_dispatch(self, x: torch.Tensor, lg: torch.Tensor, routed=None) -> torch.Tensor:
         """Expert parallel with token routing.  The ranks that hold the same rows (all of them after tensor-parallel
@@ -333,7 +372,11 @@ class FusedMoE(nn.Module):
             topk_ids = self.expert_map[topk_ids.long()]
         if self.routed_scaling_factor != 1.0:
             topk_w = topk_w * self.routed_scaling_factor
+        if self.num_identity and (self.expert_map is not None or self.eplb_state is not None):
+            raise NotImplementedError("identity experts together with expert parallelism")
         out = self.quant_method.apply(self, x, topk_w, topk_ids)
+        if self.num_identity and self.add_identity and routed is None:
+            out = (out.float() + self.identity_weight.view(-1, 1) * x.float()).to(out.dtype)
         if dispatch:
             out = dp_combine(out, meta)
         if self.reduce_results and (self.tp_size > 1 or self.ep_size > 1):

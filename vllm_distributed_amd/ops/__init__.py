@@ -367,14 +367,17 @@ def mla_cache_write(kv_c: torch.Tensor, k_pe: torch.Tensor, kc: torch.Tensor, vt
 
 def mla_attention(out: torch.Tensor, q: torch.Tensor, kc: torch.Tensor, vt: torch.Tensor, block_table: torch.Tensor,
                   seq_lens: torch.Tensor, q_start_loc: torch.Tensor, scale: float, max_query_len: int,
-                  num_splits: int = 1, kv_scale: float = 1.0, window: int = 0) -> torch.Tensor:
+                  num_splits: int = 1, kv_scale: float = 1.0, window: int = 0,
+                  sink: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal multi-query attention of q [T, H, DK] over the latent cache; out [T, H, DV] stays in latent
-    space (the caller applies the value up-projection).  Decode and (chunked) prefill are one path."""
+    space (the caller applies the value up-projection).  Decode and (chunked) prefill are one path.
+    ``sink`` fp32 [H]: exp(sink[h]) joins head h's softmax denominator, with no key and no value."""
     T, H, DK = q.shape
     DV = vt.shape[1]
     if not _dev(q):
-        out.copy_(R.mla_attention(q, kc, vt, block_table, seq_lens, q_start_loc, scale, kv_scale, window))
+        out.copy_(R.mla_attention(q, kc, vt, block_table, seq_lens, q_start_loc, scale, kv_scale, window, sink))
         return out
+    assert sink is None or (sink.dtype == torch.float32 and sink.is_contiguous() and sink.numel() == H)
     part_out = part_lse = None
     if num_splits > 1:
         part_out = torch.empty((T, H, num_splits, DV), dtype=torch.float32, device=q.device)
@@ -384,7 +387,7 @@ def mla_attention(out: torch.Tensor, q: torch.Tensor, kc: torch.Tensor, vt: torc
            seq_lens.data_ptr(), q_start_loc.data_ptr(), N.ptr(part_out), N.ptr(part_lse), seq_lens.shape[0], T, H, DK,
            DV, kc.shape[1], block_table.stride(0), num_splits, max(int(max_query_len), 1), q.stride(0),
            out.stride(0), scale, N.dt(q.dtype), int(kc.dtype == torch.float8_e4m3fn), float(kv_scale), int(window),
-           N.stream())
+           N.ptr(sink), N.stream())
     return out
 
 
@@ -892,6 +895,30 @@ def moe_grouped_sigmoid_topk(logits: torch.Tensor, bias: Optional[torch.Tensor],
     N.call("vda_moe_grouped_sigmoid_topk", w.data_ptr(), ids.data_ptr(), logits.data_ptr(), N.ptr(bias), T, E, k,
            groups, keep, int(renormalize), logits.stride(0), N.dt(logits.dtype), N.stream())
     return w, ids
+
+
+def moe_grouped_topk(logits: torch.Tensor, bias: Optional[torch.Tensor], k: int, groups: int, keep: int,
+                     renormalize: bool, scoring: str = "sigmoid", group_score: str = "top2", identity: int = 0,
+                     renorm_eps: float = 0.0):
+    """Group-limited choice in one launch.  s = sigmoid(logits) or softmax(logits) over all E outputs; choice = s + bias;
+    a group of neighbouring experts scores the sum of its two largest choices (``group_score`` "top2") or its largest
+    ("max"); the k best choices inside the ``keep`` best groups win, weighted by their plain s (divided by the
+    winners' sum + ``renorm_eps`` on request).  The last ``identity`` outputs have no expert behind them: a winner
+    among them comes back with id -1 and weight 0, and the sum of such winners' weights per token in the third
+    result.  Returns (weights f32 [T, k], ids i32 [T, k], identity weights f32 [T] or None); None when the kernel
+    does not take the sizes."""
+    T, E = logits.shape
+    if not _dev(logits) or E > 512 or k > 64 or groups > 64 or E % groups or logits.stride(1) != 1 \
+            or logits.dtype not in (torch.float32, torch.bfloat16, torch.float16):
+        return None
+    w = torch.empty((T, k), dtype=torch.float32, device=logits.device)
+    ids = torch.empty((T, k), dtype=torch.int32, device=logits.device)
+    idw = torch.empty((T,), dtype=torch.float32, device=logits.device) if identity else None
+    assert bias is None or (bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == E)
+    N.call("vda_moe_grouped_topk", w.data_ptr(), ids.data_ptr(), N.ptr(idw), logits.data_ptr(), N.ptr(bias), T, E, k,
+           groups, keep, int(renormalize), float(renorm_eps), int(scoring == "softmax"), int(group_score == "top2"),
+           int(identity), logits.stride(0), N.dt(logits.dtype), N.stream())
+    return w, ids, idw
 
 
 def group_rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, groups: int) -> torch.Tensor:
@@ -1523,6 +1550,38 @@ def residual_norms(x: torch.Tensor, y: Optional[torch.Tensor] = None, w_post: Op
     return h
 
 
+# ---- fp32 residual with parallel gated sub-layers and a norm in groups ------------------------------------------
+def gated_residual_group_norm(x: torch.Tensor, subs: list, w_next: Optional[torch.Tensor], groups: int, eps: float,
+                              out_dtype: torch.dtype) -> Optional[torch.Tensor]:
+    """One pass over the fp32 residual ``x`` [T, W]: x += sum over ``subs`` of (y + extra_w[:, None] * extra) * scale *
+    sigmoid(gate), in place -- one tuple (y, scale, gate, extra, extra_w) per sub-layer (at most two; y [T, W] in the
+    activation type, scale fp32 [W] or None, gate [T, W] pre-activations or None, extra [T, W] with extra_w fp32 [T] or
+    None) -- and, with ``w_next`` (fp32 [W]), returns the updated row normalised in ``groups`` equal consecutive parts,
+    each divided by its own root mean square, times w_next, in ``out_dtype``."""
+    T, W = x.shape
+    if not _dev(x) or (W + groups) * 4 > 60 * 1024 or len(subs) > 2:
+        return R.gated_residual_group_norm(x, subs, w_next, groups, eps, out_dtype)
+    assert x.dtype == torch.float32 and x.is_contiguous() and W % groups == 0
+    h = torch.empty((T, W), dtype=out_dtype, device=x.device) if w_next is not None else None
+    assert w_next is None or (w_next.dtype == torch.float32 and w_next.is_contiguous())
+    args = []
+    dt = out_dtype
+    for y, scale, gate, extra, extra_w in subs:
+        dt = y.dtype
+        assert y.shape == (T, W) and y.stride(1) == 1
+        assert scale is None or (scale.dtype == torch.float32 and scale.is_contiguous() and scale.numel() == W)
+        assert gate is None or (gate.dtype == y.dtype and gate.shape == (T, W) and gate.stride(1) == 1)
+        assert extra is None or (extra.dtype == y.dtype and extra.shape == (T, W) and extra.stride(1) == 1
+                                 and extra_w.dtype == torch.float32 and extra_w.is_contiguous() and extra_w.numel() == T)
+        args += [y.data_ptr(), y.stride(0), N.ptr(scale), N.ptr(gate), gate.stride(0) if gate is not None else 0,
+                 N.ptr(extra), extra.stride(0) if extra is not None else 0, N.ptr(extra_w)]
+    args += [None, 0, None, None, 0, None, 0, None] * (2 - len(subs))
+    assert h is None or not subs or h.dtype == dt
+    N.call("vda_gated_residual_group_norm", x.data_ptr(), len(subs), *args, N.ptr(w_next), N.ptr(h),
+           h.stride(0) if h is not None else 0, float(eps), int(groups), T, W, N.dt(dt), N.stream())
+    return h
+
+
 # ---- latent attention over a window -----------------------------------------------------------------------------
 def latent_norm_rope_cache(q: torch.Tensor, down: torch.Tensor, c_weight: torch.Tensor, cos_sin: torch.Tensor,
                            positions: torch.Tensor, qf: torch.Tensor, kc: Optional[torch.Tensor],
@@ -1548,17 +1607,20 @@ def latent_norm_rope_cache(q: torch.Tensor, down: torch.Tensor, c_weight: torch.
 
 def latent_window_attention(q: torch.Tensor, kc: torch.Tensor, block_table: torch.Tensor, seq_lens: torch.Tensor,
                             query_start_loc: torch.Tensor, scale: float, window: int, rank: int,
-                            max_query_len: int) -> torch.Tensor:
+                            max_query_len: int, sink: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Softmax attention of q [T, H, DK] over the latent rows kc [blocks, bs, DK] of each sequence's visible keys
-    (j <= i, and i - j < window when window > 0); returns the weighted sums of the rows' first ``rank`` values [T, H, rank]."""
+    (j <= i, and i - j < window when window > 0); returns the weighted sums of the rows' first ``rank`` values [T, H, rank].
+    ``sink`` fp32 [H]: exp(sink[h]) joins head h's softmax denominator, with no key and no value."""
     if not _dev(q):
-        return R.latent_window_attention(q, kc, block_table, seq_lens, query_start_loc, scale, window, rank)
+        return R.latent_window_attention(q, kc, block_table, seq_lens, query_start_loc, scale, window, rank, sink)
     T, H, DK = q.shape
+    assert sink is None or (sink.dtype == torch.float32 and sink.is_contiguous() and sink.numel() == H)
     assert q.is_contiguous() and kc.is_contiguous() and kc.dtype == q.dtype and kc.shape[2] == DK
     out = torch.zeros((T, H, rank), dtype=q.dtype, device=q.device)
     N.call("vda_latent_window_attention", out.data_ptr(), q.data_ptr(), kc.data_ptr(), block_table.data_ptr(),
            block_table.stride(0), seq_lens.data_ptr(), query_start_loc.data_ptr(), float(scale), int(window),
-           seq_lens.shape[0], H, DK, rank, kc.shape[1], max(int(max_query_len), 1), N.dt(q.dtype), N.stream())
+           seq_lens.shape[0], H, DK, rank, kc.shape[1], max(int(max_query_len), 1), N.ptr(sink), N.dt(q.dtype),
+           N.stream())
     return out
 
 
@@ -1637,7 +1699,9 @@ def residual_layer_norm(x: torch.Tensor, y: Optional[torch.Tensor], weight: torc
 def qk_norm_rope_cache(qkv: torch.Tensor, H: int, G: int, D: int, Dv: int, maps: int, q_weight: torch.Tensor,
                        k_weight: torch.Tensor, cos_sin: Optional[torch.Tensor], positions: torch.Tensor, rot: int,
                        eps: float, k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
-                       slot_mapping: torch.Tensor, by_map: bool = False) -> torch.Tensor:
+                       slot_mapping: torch.Tensor, by_map: bool = False, pairing: str = "halves",
+                       q_temp: Optional[tuple] = None, v_first: Optional[torch.Tensor] = None,
+                       v_lam: Optional[torch.Tensor] = None) -> torch.Tensor:
     """qkv [T, >= H*maps*D + G*maps*D + G*Dv] (queries, keys, values side by side; further columns are ignored).  Every
     D-wide map of every query / key head is divided by its root mean square, multiplied by q_weight / k_weight (fp32
     [D]), and its first ``rot`` values are rotated in the half-split layout (value i pairs with i + rot / 2; cos_sin fp32
@@ -1645,12 +1709,19 @@ def qk_norm_rope_cache(qkv: torch.Tensor, H: int, G: int, D: int, Dv: int, maps:
     maps * D] and values to v_cache [blocks, G, Dv, bs] at ``slot_mapping`` (negative: skipped).
     ``by_map`` (device kernels, for the matrix-core attention path): every map is a key head of its own, the same
     k_cache memory read as [blocks, G * maps, bs, D], and the queries come back ordered (key head, map, head inside the
-    group) as [T, H * maps, D]."""
+    group) as [T, H * maps, D].
+    ``pairing`` "neighbours": the rotation pairs value 2i with 2i + 1 (same table layout).  ``q_temp`` = (coef, every):
+    the queries at position p are multiplied by 1 + coef * ln(floor((p + 1) / every) + 1).  ``v_first`` [T, G * Dv] (row
+    stride arbitrary) with ``v_lam`` (fp32, one element): the cached values are (1 - lam) v + lam v_first."""
     used = (H + G) * maps * D + G * Dv
     if not _dev(qkv):
         assert not by_map
         return R.qk_norm_rope_cache(qkv[:, :used], H, G, D, Dv, maps, q_weight, k_weight, cos_sin, positions, rot, eps,
-                                    k_cache, v_cache, slot_mapping)
+                                    k_cache, v_cache, slot_mapping, pairing, q_temp, v_first, v_lam)
+    assert pairing in ("halves", "neighbours")
+    if v_first is not None:
+        assert v_first.dtype == qkv.dtype and v_first.stride(1) == 1 and v_first.shape[0] >= qkv.shape[0] \
+            and v_first.shape[1] == G * Dv and v_lam.dtype == torch.float32 and v_lam.numel() == 1
     T = qkv.shape[0]
     assert qkv.stride(1) == 1 and qkv.shape[1] >= used
     assert k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype and slot_mapping.dtype == torch.int64
@@ -1662,8 +1733,9 @@ def qk_norm_rope_cache(qkv: torch.Tensor, H: int, G: int, D: int, Dv: int, maps:
     qn = torch.empty((T, H * maps, D) if by_map else (T, H, maps * D), dtype=qkv.dtype, device=qkv.device)
     N.call("vda_qk_norm_rope_cache", qn.data_ptr(), qkv.data_ptr(), qkv.stride(0), q_weight.data_ptr(),
            k_weight.data_ptr(), N.ptr(cos_sin), positions.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
-           slot_mapping.data_ptr(), T, H, G, D, Dv, maps, rot, bs, float(eps), int(by_map), N.dt(qkv.dtype),
-           N.stream())
+           slot_mapping.data_ptr(), T, H, G, D, Dv, maps, rot, bs, float(eps), int(by_map),
+           int(pairing == "neighbours"), float(q_temp[0]) if q_temp else 0.0, int(q_temp[1]) if q_temp else 0,
+           N.ptr(v_first), v_first.stride(0) if v_first is not None else 0, N.ptr(v_lam), N.dt(qkv.dtype), N.stream())
     return qn
 
 
@@ -1686,7 +1758,8 @@ def masked_softmax_attention_mfma(qn: torch.Tensor, k_cache: torch.Tensor, v_cac
                                   max_decode_query_len: int, decode_num_splits: int, max_query_len: int, scale: float,
                                   H: int, window: int = 0, chunk: int = 0, sink: Optional[torch.Tensor] = None,
                                   maps: int = 1, lam: Optional[torch.Tensor] = None, eps: float = 0.0,
-                                  out_scale: float = 1.0, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+                                  out_scale: float = 1.0, gate: Optional[torch.Tensor] = None, softcap: float = 0.0,
+                                  dist_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``masked_softmax_attention`` on the matrix cores: the framework's paged attention kernels (decode form for the
     leading decode sequences of the step, tiled form for the prompts) with the window, chunk and sink as their
     options, every score map as a key head of its own that shares its group's values, and one epilogue launch for the
@@ -1699,7 +1772,9 @@ def masked_softmax_attention_mfma(qn: torch.Tensor, k_cache: torch.Tensor, v_cac
     a = torch.empty((T, Hq, D), dtype=qn.dtype, device=qn.device)
     nd, ndt, n_pre = int(num_decode_seqs), int(num_decode_tokens), int(num_prefill_seqs)
     R_ = H // G
-    kw = dict(window=int(window), sink=sink, chunk=int(chunk), v_shift=maps - 1)
+    if dist_bias is not None:
+        raise NotImplementedError("a distance bias table on the matrix-core attention path")
+    kw = dict(window=int(window), sink=sink, chunk=int(chunk), v_shift=maps - 1, softcap=float(softcap))
     cols = max(int(max_decode_query_len), 1) * R_
     if nd > 0 and (cols > 32 or (cols > 16 and D > 128)):
         raise ValueError(f"{cols} query columns per key head and step are beyond the decode form")
@@ -1729,17 +1804,22 @@ def masked_softmax_attention(qn: torch.Tensor, k_cache: torch.Tensor, v_cache: t
                              scale: float, window: int = 0, chunk: int = 0, sink: Optional[torch.Tensor] = None,
                              maps: int = 1, lam: Optional[torch.Tensor] = None, eps: float = 0.0,
                              out_scale: float = 1.0, gate: Optional[torch.Tensor] = None, max_query_len: int = 1,
-                             out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+                             out_dtype: Optional[torch.dtype] = None, softcap: float = 0.0,
+                             dist_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal softmax attention of qn [T, H, maps * D] over the paged keys and values (k_cache [blocks, G, bs, maps * D],
     v_cache [blocks, G, Dv, bs]).  Key j is visible to the query at position i when j <= i, i - j < window (window > 0)
     and j // chunk == i // chunk (chunk > 0).  ``sink`` fp32 [H]: exp(sink[h]) joins head h's denominator.  maps == 2:
     two score maps per head over the same values, o = a1 - lam * a2 (``lam``: fp32 tensor of one element), then
     o / rms(o) * out_scale over Dv.  ``gate`` [T, H * Dv] (row stride arbitrary): the result times sigmoid(gate).
+    ``softcap`` > 0: score <- softcap * tanh(score / softcap).  ``dist_bias`` fp32 [far + 1, H]: row min(i - j, far) joins
+    the (capped) scores of every head.
     Returns [T, H * Dv] in ``out_dtype`` (default: qn's type).  Scores, softmax and sums in fp32."""
     out_dtype = out_dtype or qn.dtype
     if not _dev(qn):
         return R.masked_softmax_attention(qn, k_cache, v_cache, block_table, seq_lens, query_start_loc, scale, window,
-                                          chunk, sink, maps, lam, eps, out_scale, gate, out_dtype)
+                                          chunk, sink, maps, lam, eps, out_scale, gate, out_dtype, softcap, dist_bias)
+    assert dist_bias is None or (dist_bias.dtype == torch.float32 and dist_bias.is_contiguous()
+                                 and dist_bias.dim() == 2 and dist_bias.shape[1] == qn.shape[1])
     T, H, MD = qn.shape
     G, Dv, bs = v_cache.shape[1], v_cache.shape[2], v_cache.shape[3]
     assert qn.is_contiguous() and k_cache.is_contiguous() and v_cache.is_contiguous() and MD % maps == 0
@@ -1752,5 +1832,6 @@ def masked_softmax_attention(qn: torch.Tensor, k_cache: torch.Tensor, v_cache: t
            block_table.data_ptr(), block_table.stride(0), seq_lens.data_ptr(), query_start_loc.data_ptr(),
            N.ptr(sink), N.ptr(lam), N.ptr(gate), gate.stride(0) if gate is not None else 0, float(scale), int(window),
            int(chunk), int(maps), float(eps), float(out_scale), seq_lens.shape[0], H, G, MD // maps, Dv, bs,
-           max(int(max_query_len), 1), N.dt(out_dtype), N.stream())
+           max(int(max_query_len), 1), float(softcap), N.ptr(dist_bias),
+           dist_bias.shape[0] - 1 if dist_bias is not None else 0, N.dt(out_dtype), N.stream())
     return out

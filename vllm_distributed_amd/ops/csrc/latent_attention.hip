@@ -9,7 +9,8 @@
 //                                P values (interleaved pairs, angles from an fp32 cos | sin table), write the cache
 //                                row (and, for the MFMA kernel of mla.hip, the transposed copy of c) and
 //                                qf[:, :, R:] in one launch
-//   vda_latent_window_attention  softmax(scale * qf . row) over the keys j <= i, i - j < window; scores, softmax and
+//   vda_latent_window_attention  softmax(scale * qf . row) over the keys j <= i, i - j < window (with `sink`, exp(sink[h])
+//                                joins head h's denominator without key or value); scores, softmax and
 //                                the weighted sum in fp32.  One workgroup per (sequence, tile of query tokens) walks
 //                                the visible keys in tiles through LDS with a running maximum and sum per row; keys
 //                                outside the window are never loaded.  Prompts, portions and single decoded tokens
@@ -97,7 +98,7 @@ template <typename T, int NACC>
 __global__ __launch_bounds__(256) void latent_window_attention_kernel(
     T* __restrict__ out, const T* __restrict__ qf, const T* __restrict__ kc, const int* __restrict__ block_table,
     long bt_stride, const int* __restrict__ seq_lens, const int* __restrict__ qsl, float scale, int window, int HT,
-    int HG, int DK, int R, int bs, int BQ, int BK) {
+    int HG, int DK, int R, int bs, int BQ, int BK, const float* __restrict__ sink) {
   // HT heads in all; this workgroup takes the H heads from h0 on (grid.z deals groups of HG heads)
   const int h0 = blockIdx.z * HG;
   const int H = min(HG, HT - h0);
@@ -126,7 +127,10 @@ __global__ __launch_bounds__(256) void latent_window_attention_kernel(
     const int d = e % DK, m = e / DK;             // m = i * H + h
     qs[m * Dq + d] = (m / H) < nq ? (float)qf[((long)(t0 + i0 + m / H) * HT + h0 + m % H) * DK + d] * scale : 0.f;
   }
-  for (int m = tid; m < M; m += 256) { rm[m] = -INFINITY; rl[m] = 0.f; }
+  for (int m = tid; m < M; m += 256) {
+    if (sink) { rm[m] = sink[h0 + m % H]; rl[m] = 1.f; }        // exp(sink - sink): the sink's share of the sum
+    else { rm[m] = -INFINITY; rl[m] = 0.f; }
+  }
   float acc[NACC];
 #pragma unroll
   for (int n = 0; n < NACC; ++n) acc[n] = 0.f;
@@ -207,8 +211,8 @@ __global__ __launch_bounds__(256) void latent_window_attention_kernel(
 
 VDA_EXPORT int vda_latent_window_attention(void* out, const void* qf, const void* kc, const int* block_table,
                                            long bt_stride, const int* seq_lens, const int* qsl, float scale,
-                                           int window, int S, int H, int DK, int R, int bs, int max_q, int dtype,
-                                           hipStream_t st) {
+                                           int window, int S, int H, int DK, int R, int bs, int max_q,
+                                           const float* sink, int dtype, hipStream_t st) {
   if (S <= 0 || max_q <= 0) return 0;
   if (H <= 0 || R <= 0 || R > DK) return -1;
   // tile sizes: the largest query tile (then key tile) whose accumulators fit 64 registers per thread, whose rows
@@ -242,7 +246,7 @@ VDA_EXPORT int vda_latent_window_attention(void* out, const void* qf, const void
     }                                                                                                               \
     hipLaunchKernelGGL((latent_window_attention_kernel<TT, NA>), grid, block, lds, st, (TT*)out, (const TT*)qf,     \
                        (const TT*)kc, block_table, bt_stride, seq_lens, qsl, scale, window, H, HG, DK, R, bs, BQ,   \
-                       BK);                                                                                         \
+                       BK, sink);                                                                                   \
   } while (0)
 #define L(TT)                                                                                                       \
   do {                                                                                                              \

@@ -1,6 +1,12 @@
 // Softmax attention on the paged cache with the pieces several decoder designs combine freely:
 //   * per-head RMS norms of queries and keys with a learned weight, then a rotation of the first `rot` values of a
-//     head in the half-split layout (value i pairs with value i + rot / 2), angles from an fp32 cos | sin table;
+//     head, value i paired with value i + rot / 2 (half-split) or value 2i with 2i + 1 (neighbours), angles from an
+//     fp32 cos | sin table;
+//   * a query temperature: queries at position p times 1 + coef * ln(floor((p + 1) / every) + 1);
+//   * value mixing: v <- (1 - lam) v + lam v_first with the values another layer made of the same token, before the
+//     cache write;
+//   * scores squashed by cap * tanh(score / cap); a learned bias per (query - key distance, head) from a table whose
+//     last row serves every larger distance;
 //   * key and value widths of their own (D, Dv), grouped query heads;
 //   * `maps` score maps per head over the same values (maps = 2: differential attention, o = a1 - lam * a2, divided
 //     by its root mean square over Dv and scaled);
@@ -24,18 +30,41 @@
 //                                  so a result does not depend on how a prompt was cut or batched.
 #include "common.h"
 
+// options of the per-token kernel beyond norms and rotation (zero / null: off)
+struct QkExtras {
+  int neighbours;          // rotation pairs value 2i with 2i + 1 instead of i with i + rot / 2
+  float q_coef;            // query temperature: 1 + q_coef * ln(floor((p + 1) / q_every) + 1)
+  int q_every;             //   (q_every <= 0: none)
+  const void* v_first;     // [T, G * Dv] values of the same tokens from an earlier layer, or null
+  long v_first_stride;
+  const float* v_lam;      // one value: v <- (1 - lam) v + lam v_first
+};
+
+__device__ __forceinline__ float query_temperature(const QkExtras& x, long p) {
+  if (x.q_every <= 0) return 1.f;
+  return 1.f + x.q_coef * logf((float)((p + 1) / x.q_every + 1));
+}
+
+template <typename T>
+__device__ __forceinline__ T mixed_value(const QkExtras& x, T v, long t, int e) {
+  if (!x.v_first) return v;
+  const float lam = *x.v_lam;
+  return (T)((1.f - lam) * (float)v + lam * (float)((const T*)x.v_first)[t * x.v_first_stride + e]);
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void qk_norm_rope_cache_kernel(
     T* __restrict__ qn, const T* __restrict__ qkv, long qkv_stride, const float* __restrict__ q_w,
     const float* __restrict__ k_w, const float* __restrict__ cos_sin, const long* __restrict__ positions,
     T* __restrict__ k_cache, T* __restrict__ v_cache, const long* __restrict__ slot_mapping, int H, int G, int D,
-    int Dv, int maps, int rot, int bs, float eps, int by_map) {
+    int Dv, int maps, int rot, int bs, float eps, int by_map, const QkExtras x) {
   const long t = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const T* row = qkv + t * qkv_stride;
   const int half = rot / 2;
   const float* cs = rot > 0 ? cos_sin + positions[t] * (long)rot : nullptr;
   const long slot = slot_mapping[t];
+  const float qt = query_temperature(x, positions[t]);
   const int nq = H * maps, nk = G * maps;
   // one wave per D-wide unit: the query maps first, then the key maps
   for (int u = wave; u < nq + nk; u += 4) {
@@ -67,19 +96,20 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_kernel(
     for (int d = lane; d < D; d += 64) {
       float v = (float)src[d] * rs * w[d];
       if (d < rot) {
-        const int i = d < half ? d : d - half;
-        const int pd = d < half ? d + half : d - half;
+        const bool first = x.neighbours ? !(d & 1) : d < half;
+        const int i = x.neighbours ? d >> 1 : (d < half ? d : d - half);
+        const int pd = x.neighbours ? d ^ 1 : (d < half ? d + half : d - half);
         const float o = (float)src[pd] * rs * w[pd];
         const float co = cs[i], si = cs[half + i];
-        v = d < half ? v * co - o * si : v * co + o * si;
+        v = first ? v * co - o * si : v * co + o * si;
       }
-      dst[d] = (T)v;
+      dst[d] = (T)(is_q ? v * qt : v);
     }
   }
   if (slot >= 0) {
     const T* vsrc = row + (long)(nq + nk) * D;
     T* vdst = v_cache + (slot / bs) * (long)G * Dv * bs + slot % bs;      // [blocks, G, Dv, bs]
-    for (int e = tid; e < G * Dv; e += 256) vdst[(long)e * bs] = vsrc[e];
+    for (int e = tid; e < G * Dv; e += 256) vdst[(long)e * bs] = mixed_value<T>(x, vsrc[e], t, e);
   }
 }
 
@@ -91,7 +121,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_vec_kernel(
     T* __restrict__ qn, const T* __restrict__ qkv, long qkv_stride, const float* __restrict__ q_w,
     const float* __restrict__ k_w, const float* __restrict__ cos_sin, const long* __restrict__ positions,
     T* __restrict__ k_cache, T* __restrict__ v_cache, const long* __restrict__ slot_mapping, int H, int G, int Dv,
-    int maps, int rot, int bs, float eps, int by_map) {
+    int maps, int rot, int bs, float eps, int by_map, const QkExtras xo) {
   using V8 = typename Vec<T>::v8;
   constexpr int D = LPU * 8, UPB = 256 / LPU;
   const long t = blockIdx.x;
@@ -100,6 +130,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_vec_kernel(
   const int half = rot / 2, hl = half / 8;          // partner lane distance
   const float* cs = rot > 0 ? cos_sin + positions[t] * (long)rot : nullptr;
   const long slot = slot_mapping[t];
+  const float qt = query_temperature(xo, positions[t]);
   const int nq = H * maps, nk = G * maps, total = nq + nk;
   for (int u0 = 0; u0 < total; u0 += UPB) {
     const int u = u0 + tid / LPU;
@@ -116,7 +147,18 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_vec_kernel(
     const float rs = 1.f / sqrtf(ss / (float)D + eps);
 #pragma unroll
     for (int i = 0; i < 8; ++i) x[i] *= rs * w[i];
-    if (rot > 0) {                                   // uniform
+    if (rot > 0 && xo.neighbours) {                  // uniform: a pair sits in one lane
+      if (d0 < rot) {
+        const float* cp = cs + d0 / 2;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float co = cp[i], si = cp[half + i];
+          const float a = x[2 * i], b = x[2 * i + 1];
+          x[2 * i] = a * co - b * si;
+          x[2 * i + 1] = b * co + a * si;
+        }
+      }
+    } else if (rot > 0) {                            // uniform
       const bool lowh = d0 < half, turn = d0 < rot;
       const int partner = (tid & 63) + (lowh ? hl : -hl);
       const float* cp = cs + (lowh ? d0 : d0 - half);
@@ -145,30 +187,36 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_vec_kernel(
       dst = by_map ? k_cache + (((slot / bs) * nk + uk) * (long)bs + slot % bs) * (long)D
                    : k_cache + (((slot / bs) * G + g) * (long)bs + slot % bs) * (long)(maps * D) + (long)mp * D;
     }
+    const float mul = is_q ? qt : 1.f;
     V8 o8;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) o8[i] = (T)x[i];
+    for (int i = 0; i < 8; ++i) o8[i] = (T)(x[i] * mul);
     st16<V8>(dst + d0, o8);
   }
   if (slot >= 0) {
     const T* vsrc = row + (long)total * D;
     T* vdst = v_cache + (slot / bs) * (long)G * Dv * bs + slot % bs;      // [blocks, G, Dv, bs]
-    for (int e = tid; e < G * Dv; e += 256) vdst[(long)e * bs] = vsrc[e];
+    for (int e = tid; e < G * Dv; e += 256) vdst[(long)e * bs] = mixed_value<T>(xo, vsrc[e], t, e);
   }
 }
 
 VDA_EXPORT int vda_qk_norm_rope_cache(void* qn, const void* qkv, long qkv_stride, const float* q_w, const float* k_w,
                                       const float* cos_sin, const long* positions, void* k_cache, void* v_cache,
                                       const long* slot_mapping, int T, int H, int G, int D, int Dv, int maps, int rot,
-                                      int bs, float eps, int by_map, int dtype, hipStream_t st) {
+                                      int bs, float eps, int by_map, int neighbours, float q_coef, int q_every,
+                                      const void* v_first, long v_first_stride, const float* v_lam, int dtype,
+                                      hipStream_t st) {
   if (T <= 0) return 0;
-  if (rot < 0 || rot > D || (rot & 1) || maps < 1 || (rot > 0 && !cos_sin)) return -1;
-  const bool vec = (D == 32 || D == 64 || D == 128 || D == 256) && (rot / 2) % 8 == 0 && qkv_stride % 8 == 0 &&
+  if (rot < 0 || rot > D || (rot & 1) || maps < 1 || (rot > 0 && !cos_sin) || (v_first && !v_lam)) return -1;
+  const QkExtras xo{neighbours, q_coef, q_every, v_first, v_first_stride, v_lam};
+  // half-split pairs: the partner sits rot / 16 lanes away; neighbours: inside the lane's own eight values
+  const bool vec = (D == 32 || D == 64 || D == 128 || D == 256) && (neighbours ? rot % 8 == 0 : (rot / 2) % 8 == 0) &&
+                   qkv_stride % 8 == 0 &&
                    ((uintptr_t)qkv % 32 == 0) && ((uintptr_t)qn % 32 == 0) && ((uintptr_t)k_cache % 32 == 0);
   if (vec) {
 #define LV2(TT, LL) hipLaunchKernelGGL((qk_norm_rope_cache_vec_kernel<TT, LL>), dim3(T), dim3(256), 0, st, (TT*)qn,    \
                                        (const TT*)qkv, qkv_stride, q_w, k_w, cos_sin, positions, (TT*)k_cache,          \
-                                       (TT*)v_cache, slot_mapping, H, G, Dv, maps, rot, bs, eps, by_map)
+                                       (TT*)v_cache, slot_mapping, H, G, Dv, maps, rot, bs, eps, by_map, xo)
 #define LV(TT) do { if (D == 32) LV2(TT, 4); else if (D == 64) LV2(TT, 8); else if (D == 128) LV2(TT, 16); else LV2(TT, 32); } while (0)
     if (dtype == VDA_BF16) LV(bf16_t);
     else if (dtype == VDA_F16) LV(f16_t);
@@ -181,7 +229,7 @@ VDA_EXPORT int vda_qk_norm_rope_cache(void* qn, const void* qkv, long qkv_stride
   }
 #define L(TT) hipLaunchKernelGGL((qk_norm_rope_cache_kernel<TT>), dim3(T), dim3(256), 0, st, (TT*)qn, (const TT*)qkv,  \
                                  qkv_stride, q_w, k_w, cos_sin, positions, (TT*)k_cache, (TT*)v_cache, slot_mapping,  \
-                                 H, G, D, Dv, maps, rot, bs, eps, by_map)
+                                 H, G, D, Dv, maps, rot, bs, eps, by_map, xo)
   if (dtype == VDA_BF16) L(bf16_t);
   else if (dtype == VDA_F16) L(f16_t);
   else if (dtype == VDA_F32) L(float);
@@ -204,7 +252,9 @@ struct MaskedAttnArgs {
   const float* lam;          // one value (maps == 2)
   const void* gate;          // [T, H * Dv] pre-activations or null
   long gate_stride;
-  float scale, eps, out_scale;
+  const float* dist_bias;    // [far + 1, H] or null: row min(i - j, far) joins the scores
+  int far;
+  float scale, eps, out_scale, softcap;
   int window, chunk, maps;
   int H, G, D, Dv, bs;
   int HG;                    // heads per workgroup (of the H / G that share a key / value head)
@@ -304,6 +354,8 @@ __global__ __launch_bounds__(256) void masked_softmax_attention_kernel(const Mas
         const float* kp = ks + jj * Kq + (m % maps) * D;
         sv = 0.f;
         for (int d = 0; d < D; ++d) sv += qp[d] * kp[d];
+        if (a.softcap > 0.f) sv = a.softcap * tanhf(sv / a.softcap);
+        if (a.dist_bias) sv += a.dist_bias[(long)min(pi - j, a.far) * a.H + h0 + (m / maps) % HN];
       }
       sc[m * RS + jj] = sv;
     }
@@ -390,9 +442,12 @@ VDA_EXPORT int vda_masked_softmax_attention(void* out, const void* qn, const voi
                                             const int* qsl, const float* sink, const float* lam, const void* gate,
                                             long gate_stride, float scale, int window, int chunk, int maps, float eps,
                                             float out_scale, int S, int H, int G, int D, int Dv, int bs, int max_q,
-                                            int dtype, hipStream_t st) {
+                                            float softcap, const float* dist_bias, int far, int dtype,
+                                            hipStream_t st) {
   if (S <= 0 || max_q <= 0) return 0;
-  if (H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0 || maps < 1 || maps > 2 || (maps == 2 && !lam)) return -1;
+  if (H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0 || maps < 1 || maps > 2 || (maps == 2 && !lam) ||
+      (dist_bias && far < 0))
+    return -1;
   // tile sizes: the largest query tile (then key tile) whose accumulators fit 64 registers per thread, whose rows
   // fit one workgroup and whose tiles fit 96 KiB of LDS; single decoded tokens take a one-token tile; the heads of
   // a group are dealt to several workgroups when one token's heads alone are too many for that
@@ -424,6 +479,7 @@ VDA_EXPORT int vda_masked_softmax_attention(void* out, const void* qn, const voi
   a.bt_stride = bt_stride; a.seq_lens = seq_lens; a.qsl = qsl; a.sink = sink; a.lam = lam; a.gate = gate;
   a.gate_stride = gate_stride; a.scale = scale; a.eps = eps; a.out_scale = out_scale; a.window = window;
   a.chunk = chunk; a.maps = maps; a.H = H; a.G = G; a.D = D; a.Dv = Dv; a.bs = bs; a.HG = HG; a.BQ = BQ; a.BK = BK;
+  a.softcap = softcap; a.dist_bias = dist_bias; a.far = far;
   dim3 grid((max_q + BQ - 1) / BQ, S, G * ((R + HG - 1) / HG)), block(256);
 #define L2(TT, NA)                                                                                                  \
   do {                                                                                                              \

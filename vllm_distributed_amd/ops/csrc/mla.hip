@@ -85,6 +85,7 @@ struct MlaParams {
   float scale;              // softmax scale, times the cache scale for an fp8 cache
   float v_scale;            // 1, or the cache scale for an fp8 cache
   int window;               // > 0: a query at position i sees the keys j with 0 <= i - j < window
+  const float* sink;        // [H] or null: exp(sink[h]) joins head h's softmax denominator, with no key and no value
   int wave_cols;            // 1: every wave takes 16 columns of its own over all keys (prompts: neighbouring tokens
                             //    walk the same keys at the same time, so the rows come from the cache near the CU);
                             // 0: the 4 waves share 16 columns and split the keys (few query tokens)
@@ -140,7 +141,10 @@ __global__ __launch_bounds__(256) void mla_attention_kernel(MlaParams p) {
   const int a0 = step_lo + blockIdx.z * per;
   step_hi = min(step_hi, a0 + per);
 
-  float m = -INFINITY, l = 0.f;
+  // a sink is a score without key or value: the running maximum starts there and the sum with its weight of one,
+  // in one lane group, one wave and one key partition, so that it counts once
+  const bool own_sink = p.sink && valid && blockIdx.z == 0 && (p.wave_cols || wave == 0);
+  float m = own_sink ? p.sink[head] * 1.4426950408889634f : -INFINITY, l = (own_sink && g == 0) ? 1.f : 0.f;
   f32x4 acc[NT];
 #pragma unroll
   for (int n = 0; n < NT; ++n) acc[n] = f32x4{0, 0, 0, 0};
@@ -302,7 +306,8 @@ __global__ __launch_bounds__(256) void mla_prefill_kernel(MlaParams p) {
   const int wg_hi = (ctx + t_last + 1 + 31) / 32;
   const int wg_lo = p.window > 0 ? max(ctx + t_first + 1 - p.window, 0) / 32 : 0;
 
-  float m = -INFINITY, l = 0.f;
+  const bool own_sink = p.sink && valid;               // see mla_attention_kernel
+  float m = own_sink ? p.sink[head] * 1.4426950408889634f : -INFINITY, l = (own_sink && g == 0) ? 1.f : 0.f;
   f32x4 acc[NT];
 #pragma unroll
   for (int n = 0; n < NT; ++n) acc[n] = f32x4{0, 0, 0, 0};
@@ -481,7 +486,7 @@ VDA_EXPORT int vda_mla_attention(void* out, const void* q, const void* kc, const
                                  const int* seq_lens, const int* q_start_loc, float* part_out, float* part_lse,
                                  int S, int T_tokens, int H, int DK, int DV, int BS, int max_blocks, int nsplit,
                                  int max_q, long q_stride, long out_stride, float scale, int dtype, int kv_fp8,
-                                 float kv_scale, int window, hipStream_t st) {
+                                 float kv_scale, int window, const float* sink, hipStream_t st) {
   if (S <= 0 || T_tokens <= 0) return 0;
   if (!vda_mla_supported(DK, DV) || BS % 8 || nsplit < 1 || nsplit > 64 || (nsplit > 1 && (!part_out || !part_lse)))
     return -1;      // (the reduce kernel keeps one partition per lane)
@@ -492,6 +497,7 @@ VDA_EXPORT int vda_mla_attention(void* out, const void* q, const void* kc, const
   p.q_stride = q_stride; p.out_stride = out_stride;
   p.scale = scale * (kv_fp8 ? kv_scale : 1.f); p.v_scale = kv_fp8 ? kv_scale : 1.f;
   p.window = window > 0 ? window : 0;
+  p.sink = sink;
   p.wave_cols = (nsplit == 1 && (long)max_q * H >= 64) ? 1 : 0;
   const bool f8 = kv_fp8 != 0;
   int rc = 0;

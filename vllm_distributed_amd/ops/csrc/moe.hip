@@ -72,15 +72,20 @@ __global__ __launch_bounds__(256) void moe_topk_softmax_kernel(float* __restrict
   }
 }
 
-// Group-limited choice with sigmoid scores and a selection bias (DeepSeek-V3 style routing), one wave per token:
-//   s = sigmoid(logit);  choice = s + bias;  experts form `groups` equal groups of neighbours, a group's score is the
-//   sum of its two largest choice scores (its largest when it has one member); only the `keep` best groups stay in the
-//   race (the others count as minus infinity); the k largest choice scores win and are weighted by their plain s
-//   (divided by the winners' sum when renorm is set).
+// Group-limited choice with a selection bias (DeepSeek-V3 style routing), one wave per token:
+//   s = sigmoid(logit), or softmax(logits) over all E outputs (`softmax`);  choice = s + bias;  experts form `groups`
+//   equal groups of neighbours, a group's score is the sum of its two largest choice scores (`top2`; its largest when
+//   it has one member) or its largest one; only the `keep` best groups stay in the race (the others count as minus
+//   infinity); the k largest choice scores win and are weighted by their plain s (divided by the winners' sum +
+//   renorm_eps when renorm is set).
+//   The last `identity` of the E outputs have no expert behind them (their output is the layer's input itself):
+//   a winner among them gets the id -1, which every expert kernel skips, and the sum of such winners' weights
+//   goes to id_w[t].
 template <typename T>
 __global__ __launch_bounds__(256) void moe_grouped_sigmoid_topk_kernel(
     float* __restrict__ topk_w, int* __restrict__ topk_id, const T* __restrict__ logits,
-    const float* __restrict__ bias, int num_tokens, int E, int k, int groups, int keep, int renorm, long stride) {
+    const float* __restrict__ bias, int num_tokens, int E, int k, int groups, int keep, int renorm, long stride,
+    int softmax, int top2, int identity, float renorm_eps, float* __restrict__ id_w) {
   const int lane = threadIdx.x & 63;
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= num_tokens) return;
@@ -90,8 +95,28 @@ __global__ __launch_bounds__(256) void moe_grouped_sigmoid_topk_kernel(
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
     const int e = lane + 64 * i;
-    const float z = e < E ? (float)logits[(long)t * stride + e] : 0.f;
-    s[i] = 1.f / (1.f + expf(-z));
+    const float z = e < E ? (float)logits[(long)t * stride + e] : (softmax ? -INFINITY : 0.f);
+    s[i] = softmax ? z : 1.f / (1.f + expf(-z));
+  }
+  if (softmax) {
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) mx = fmaxf(mx, s[i]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      s[i] = lane + 64 * i < E ? expf(s[i] - mx) : 0.f;
+      sum += s[i];
+    }
+    sum = wave_sum(sum);
+#pragma unroll
+    for (int i = 0; i < PER; ++i) s[i] /= sum;
+  }
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int e = lane + 64 * i;
     c[i] = e < E ? s[i] + (bias ? bias[e] : 0.f) : -INFINITY;
     if (!(c[i] == c[i])) c[i] = -INFINITY;          // NaN logits (warm-up runs over empty contexts)
   }
@@ -115,7 +140,7 @@ __global__ __launch_bounds__(256) void moe_grouped_sigmoid_topk_kernel(
         m2 = fmaxf(fminf(m1, a1), fmaxf(m2, a2));
         m1 = hi;
       }
-      const float sc = gs > 1 ? m1 + m2 : m1;
+      const float sc = (gs > 1 && top2) ? m1 + m2 : m1;
       if (lane == g) gscore = sc;
     }
     unsigned long long allowed = 0ull;
@@ -160,23 +185,29 @@ __global__ __launch_bounds__(256) void moe_grouped_sigmoid_topk_kernel(
     picked += bs;
     if (lane == j) { my_w = bs; my_id = bi; }
   }
+  const float scale = renorm ? (picked + renorm_eps > 0.f ? 1.f / (picked + renorm_eps) : 0.f) : 1.f;
+  const bool ident = lane < k && my_id >= E - identity;
   if (lane < k) {
-    const float scale = renorm ? (picked > 0.f ? 1.f / picked : 0.f) : 1.f;
-    topk_w[(long)t * k + lane] = my_w * scale;
-    topk_id[(long)t * k + lane] = my_id;
+    topk_w[(long)t * k + lane] = ident ? 0.f : my_w * scale;
+    topk_id[(long)t * k + lane] = ident ? -1 : my_id;
+  }
+  if (id_w) {
+    const float iw = wave_sum(ident ? my_w * scale : 0.f);
+    if (lane == 0) id_w[t] = iw;
   }
 }
 
-VDA_EXPORT int vda_moe_grouped_sigmoid_topk(float* topk_w, int* topk_id, const void* logits, const float* bias,
-                                            int num_tokens, int E, int k, int groups, int keep, int renorm,
-                                            long stride, int dtype, hipStream_t st) {
+static int launch_grouped_topk(float* topk_w, int* topk_id, const void* logits, const float* bias, int num_tokens,
+                               int E, int k, int groups, int keep, int renorm, long stride, int softmax, int top2,
+                               int identity, float renorm_eps, float* id_w, int dtype, hipStream_t st) {
   if (num_tokens <= 0) return 0;
   if (E < 1 || E > 512 || k < 1 || k > 64 || k > E || groups < 1 || groups > 64 || E % groups || keep < 1 ||
-      keep > groups)
+      keep > groups || identity < 0 || identity > E || (identity > 0 && !id_w))
     return -1;
   dim3 grid((num_tokens + 3) / 4), block(256);
 #define L(TT) hipLaunchKernelGGL((moe_grouped_sigmoid_topk_kernel<TT>), grid, block, 0, st, topk_w, topk_id,          \
-                                 (const TT*)logits, bias, num_tokens, E, k, groups, keep, renorm, stride)
+                                 (const TT*)logits, bias, num_tokens, E, k, groups, keep, renorm, stride, softmax,    \
+                                 top2, identity, renorm_eps, id_w)
   if (dtype == VDA_BF16) L(bf16_t);
   else if (dtype == VDA_F16) L(f16_t);
   else if (dtype == VDA_F32) L(float);
@@ -185,6 +216,21 @@ VDA_EXPORT int vda_moe_grouped_sigmoid_topk(float* topk_w, int* topk_id, const v
   VDA_CHECK_LAUNCH();
   return 0;
 }
+
+VDA_EXPORT int vda_moe_grouped_sigmoid_topk(float* topk_w, int* topk_id, const void* logits, const float* bias,
+                                            int num_tokens, int E, int k, int groups, int keep, int renorm,
+                                            long stride, int dtype, hipStream_t st) {
+  return launch_grouped_topk(topk_w, topk_id, logits, bias, num_tokens, E, k, groups, keep, renorm, stride, 0, 1, 0,
+                             0.f, nullptr, dtype, st);
+}
+
+VDA_EXPORT int vda_moe_grouped_topk(float* topk_w, int* topk_id, float* id_w, const void* logits, const float* bias,
+                                    int num_tokens, int E, int k, int groups, int keep, int renorm, float renorm_eps,
+                                    int softmax, int top2, int identity, long stride, int dtype, hipStream_t st) {
+  return launch_grouped_topk(topk_w, topk_id, logits, bias, num_tokens, E, k, groups, keep, renorm, stride, softmax,
+                             top2, identity, renorm_eps, id_w, dtype, st);
+}
+
 
 VDA_EXPORT int vda_moe_topk_softmax(float* topk_w, int* topk_id, const void* logits, int num_tokens, int E, int k,
                                     int renorm, long stride, int dtype, hipStream_t st) {

@@ -293,6 +293,123 @@ VDA_EXPORT int vda_group_rms_norm(void* out, long o_stride, const void* x, long 
   return 0;
 }
 
+// Parallel sub-layers behind per-channel gates over an fp32 residual, and the next norm in groups, in ONE pass:
+//   x[t] += sum over the sub-layers of (y + extra_w[t] * extra) * scale * sigmoid(gate)      (in place, fp32)
+//   h[t]  = x[t] / rms_g(x[t]) * w_next    with rms_g the root mean square of the value's own part, the row being
+//           split into `groups` equal consecutive parts
+// Every piece is optional: no sub-layer at all is the stack's first or last norm, no h is the last residual update.
+// One workgroup per token; the updated row waits in LDS for its parts' sums.
+struct GatedSub {
+  const void* y;        // [T, W] the sub-layer's output
+  long y_stride;
+  const float* scale;   // [W] or null
+  const void* gate;     // [T, W] pre-activations of the sigmoid gate, or null
+  long gate_stride;
+  const void* extra;    // [T, W] or null: joins y times extra_w[t]
+  long extra_stride;
+  const float* extra_w; // [T]
+};
+struct GatedResidualArgs {
+  float* x;
+  GatedSub sub[2];
+  int nsub;
+  const float* w_next;
+  void* h;
+  long h_stride;
+  float eps;
+  int W, groups;
+};
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void gated_residual_group_norm_kernel(const GatedResidualArgs a) {
+  extern __shared__ float row[];          // the updated residual row, then one factor per part
+  const long t = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int W = a.W;
+  float* xr = a.x + t * W;
+  float* rs = row + W;
+  for (int c = tid * VEC; c < W; c += 256 * VEC) {
+    float v[VEC], add[VEC];
+    if (VEC == 4) {
+      const f32x4 q = *reinterpret_cast<const f32x4*>(xr + c);
+      v[0] = q[0]; v[1 % VEC] = q[1]; v[2 % VEC] = q[2]; v[3 % VEC] = q[3];
+    } else {
+      v[0] = xr[c];
+    }
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) add[i] = 0.f;
+    for (int sI = 0; sI < a.nsub; ++sI) {
+      const GatedSub& u = a.sub[sI];
+      const T* yr = (const T*)u.y + t * u.y_stride + c;
+      const T* gr = u.gate ? (const T*)u.gate + t * u.gate_stride + c : nullptr;
+      const T* er = u.extra ? (const T*)u.extra + t * u.extra_stride + c : nullptr;
+      const float ew = u.extra ? u.extra_w[t] : 0.f;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        float f = (float)yr[i];
+        if (er) f += ew * (float)er[i];
+        if (u.scale) f *= u.scale[c + i];
+        if (gr) f *= 1.f / (1.f + expf(-(float)gr[i]));
+        add[i] += f;
+      }
+    }
+    if (a.nsub > 0) {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) v[i] += add[i];
+      if (VEC == 4) *reinterpret_cast<f32x4*>(xr + c) = f32x4{v[0], v[1 % VEC], v[2 % VEC], v[3 % VEC]};
+      else xr[c] = v[0];
+    }
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) row[c + i] = v[i];
+  }
+  if (!a.h) return;
+  __syncthreads();
+  const int part = W / a.groups;
+  for (int g = wave; g < a.groups; g += 4) {
+    const float* pr = row + (long)g * part;
+    float ss = 0.f;
+    for (int c = lane; c < part; c += 64) ss += pr[c] * pr[c];
+    ss = wave_sum(ss);
+    if (lane == 0) rs[g] = 1.f / sqrtf(ss / (float)part + a.eps);
+  }
+  __syncthreads();
+  T* hr = (T*)a.h + t * a.h_stride;
+  for (int c = tid * VEC; c < W; c += 256 * VEC) {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) hr[c + i] = (T)(row[c + i] * rs[(c + i) / part] * a.w_next[c + i]);
+  }
+}
+
+VDA_EXPORT int vda_gated_residual_group_norm(
+    float* x, int nsub, const void* y0, long y0_stride, const float* s0, const void* g0, long g0_stride,
+    const void* e0, long e0_stride, const float* ew0, const void* y1, long y1_stride, const float* s1, const void* g1,
+    long g1_stride, const void* e1, long e1_stride, const float* ew1, const float* w_next, void* h, long h_stride,
+    float eps, int groups, int T, int W, int dtype, hipStream_t st) {
+  if (T <= 0 || (nsub == 0 && !h)) return 0;
+  if (nsub < 0 || nsub > 2 || (nsub > 0 && !y0) || (nsub > 1 && !y1) || (h && !w_next) || groups < 1 || W % groups ||
+      (e0 && !ew0) || (e1 && !ew1))
+    return -1;
+  const size_t lds = ((size_t)W + groups) * 4;
+  if (lds > 60 * 1024) return -2;
+  GatedResidualArgs a;
+  a.x = x; a.nsub = nsub; a.w_next = w_next; a.h = h; a.h_stride = h_stride; a.eps = eps; a.W = W; a.groups = groups;
+  a.sub[0] = GatedSub{y0, y0_stride, s0, g0, g0_stride, e0, e0_stride, ew0};
+  a.sub[1] = GatedSub{y1, y1_stride, s1, g1, g1_stride, e1, e1_stride, ew1};
+  bool vec = W % 4 == 0 && h_stride % 4 == 0;
+  for (int i = 0; i < nsub; ++i)
+    vec = vec && a.sub[i].y_stride % 4 == 0 && a.sub[i].gate_stride % 4 == 0 && a.sub[i].extra_stride % 4 == 0;
+#define L2(TT, VV) hipLaunchKernelGGL((gated_residual_group_norm_kernel<TT, VV>), dim3(T), dim3(256), lds, st, a)
+#define L(TT) do { if (vec) L2(TT, 4); else L2(TT, 1); } while (0)
+  if (dtype == VDA_BF16) L(bf16_t);
+  else if (dtype == VDA_F16) L(f16_t);
+  else if (dtype == VDA_F32) L(float);
+  else return -3;
+#undef L
+#undef L2
+  VDA_CHECK_LAUNCH();
+  return 0;
+}
+
 VDA_EXPORT int vda_residual_norms(float* x, const void* y, long y_stride, const float* w_post, const float* w_pre,
                                   void* h, long h_stride, float eps, float off, int T, int W, int dtype,
                                   hipStream_t st) {

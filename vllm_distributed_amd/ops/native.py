@@ -61,16 +61,19 @@ _SIGS = {
     "vda_moe_align": [P, P, P, I, I, P],
     "vda_residual_norms": [P, P, L, P, P, P, L, F, F, I, I, I, P],
     "vda_latent_norm_rope_cache": [P, L, P, L, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
-    "vda_latent_window_attention": [P, P, P, P, L, P, P, F, I, I, I, I, I, I, I, I, P],
+    "vda_latent_window_attention": [P, P, P, P, L, P, P, F, I, I, I, I, I, I, I, P, I, P],
     "vda_mlstm": [P, L, P, P, L, P, P, P, P, P, P, P, P, L, I, I, I, I, I, I, F, F, I, P],
     "vda_moe_grouped_sigmoid_topk": [P, P, P, P, I, I, I, I, I, I, L, I, P],
+    "vda_moe_grouped_topk": [P, P, P, P, P, I, I, I, I, I, I, F, I, I, I, L, I, P],
+    "vda_gated_residual_group_norm": [P, I, P, L, P, P, L, P, L, P, P, L, P, P, L, P, L, P, P, P, L, F, I, I, I, I, P],
     "vda_group_rms_norm": [P, L, P, L, P, F, I, I, I, I, I, P],
     "vda_moe_pairs": [P, L, P, P, L, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
     "vda_residual_layer_norm": [P, P, L, P, P, P, L, F, I, I, I, P, L, P, L, P],
     "vda_fp32_rows_dot": [P, P, L, P, P, I, I, I, I, P],
-    "vda_qk_norm_rope_cache": [P, P, L, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, I, I, P],
+    "vda_qk_norm_rope_cache": [P, P, L, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, I, I, F, I, P, L, P, I, P],
     "vda_map_combine": [P, P, P, P, L, I, I, I, I, I, F, F, I, P],
-    "vda_masked_softmax_attention": [P, P, P, P, P, L, P, P, P, P, P, L, F, I, I, I, F, F, I, I, I, I, I, I, I, I, P],
+    "vda_masked_softmax_attention": [P, P, P, P, P, L, P, P, P, P, P, L, F, I, I, I, F, F, I, I, I, I, I, I, I, F, P, I,
+                                     I, P],
     "vda_moe_gate_up": [P, P, P, P, P, P, I, I, I, I, I, L, I, I, I, I, F, P],
     "vda_moe_down": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
     "vda_moe_up_act": [P, P, P, P, P, I, I, I, I, I, L, I, I, I, P],
@@ -92,7 +95,7 @@ _SIGS = {
     "vda_cb4_dequant_post": [P, P, P, P, I, I, I, I, I, P],
     "vda_w8_dequant": [P, P, P, P, I, I, I, I, P],
     "vda_mla_cache_write": [P, P, P, P, P, I, I, I, I, L, L, I, I, F, P],
-    "vda_mla_attention": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, L, L, F, I, I, F, I, P],
+    "vda_mla_attention": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, L, L, F, I, I, F, I, P, P],
     "vda_mla_supported": [I, I],
     "vda_lora_shrink": [P, P, P, P, I, I, I, L, I, P],
     "vda_lora_expand": [P, P, P, P, I, I, I, L, I, P],

@@ -553,7 +553,8 @@ def mla_cache_write(kv_c, k_pe, kc, vt, slot_mapping, kv_scale=1.0):
         vt[b, :, o] = kv_c[t].to(vt.dtype)
 
 
-def mla_attention(q, kc, vt, block_table, seq_lens, q_start_loc, scale, kv_scale=1.0, window=0):
+def mla_attention(q, kc, vt, block_table, seq_lens, q_start_loc, scale, kv_scale=1.0, window=0, sink=None):
+    """``sink`` fp32 [H]: exp(sink[h]) joins head h's softmax denominator (no key, no value)."""
     T, H, DK = q.shape
     DV, BS = vt.shape[1], kc.shape[1]
     if kc.dtype != torch.float8_e4m3fn:
@@ -576,8 +577,18 @@ def mla_attention(q, kc, vt, block_table, seq_lens, q_start_loc, scale, kv_scale
         sc = sc.masked_fill(pos >= lim, float("-inf"))
         if window > 0:
             sc = sc.masked_fill(pos < lim - window, float("-inf"))
-        out[a:b] = torch.einsum("nhl,ld->nhd", torch.softmax(sc, dim=-1), V).to(q.dtype)
+        out[a:b] = torch.einsum("nhl,ld->nhd", softmax_with_sink(sc, sink.view(1, H, 1) if sink is not None else None),
+                                V).to(q.dtype)
     return out
+
+
+def softmax_with_sink(sc, sink=None):
+    """Softmax over the last dimension; ``sink`` (broadcastable to sc[..., :1]) adds exp(sink) to the denominator."""
+    if sink is None:
+        return torch.softmax(sc, dim=-1)
+    mx = torch.maximum(sc.max(-1, keepdim=True).values, sink.float())
+    e = torch.exp(sc - mx)
+    return e / (e.sum(-1, keepdim=True) + torch.exp(sink.float() - mx))
 
 
 # ---- residual streams (hyper-connections) ---------------------------------------------------------
@@ -703,6 +714,31 @@ def residual_norms(x, y, w_post, w_pre, eps: float, out_dtype, gain_offset: floa
     return (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * (gain_offset + w_pre.float())).to(out_dtype)
 
 
+def gated_residual_group_norm(x, subs, w_next, groups: int, eps: float, out_dtype):
+    """x fp32 [T, W], in place: x += sum over ``subs`` of y * scale * sigmoid(gate), one tuple (y, scale, gate, extra,
+    extra_w) per sub-layer (scale fp32 [W] or None, gate [T, W] pre-activations or None, extra [T, W] with extra_w fp32
+    [T] or None: y + extra_w[:, None] * extra takes y's place); the sub-layers' terms are summed before they join x.
+    With ``w_next`` returns every one of ``groups`` equal parts of the updated row divided by its own root mean square,
+    times w_next, in ``out_dtype``."""
+    total = None
+    for y, scale, gate, extra, extra_w in subs:
+        f = y.float()
+        if extra is not None:
+            f = f + extra_w.float().view(-1, 1) * extra.float()
+        if scale is not None:
+            f = f * scale.float()
+        if gate is not None:
+            f = f * torch.sigmoid(gate.float())
+        total = f if total is None else total + f
+    if total is not None:
+        x += total
+    if w_next is None:
+        return None
+    T, W = x.shape
+    p = x.view(T, groups, W // groups)
+    return ((p * torch.rsqrt(p.pow(2).mean(-1, keepdim=True) + eps)).view(T, W) * w_next.float()).to(out_dtype)
+
+
 # ---- latent attention over a window: cache write and attention ----------------------------------------------
 def rotate_interleaved(x, cos, sin):
     """x [..., 2n] as pairs (x[2i], x[2i+1]) turned by the angles whose cos / sin [..., n] are given (fp32)."""
@@ -735,9 +771,10 @@ def latent_norm_rope_cache(q, down, c_weight, cos_sin, positions, qf, kc, slot_m
             vt[sl // bs, :, sl % bs] = c[ok].to(vt.dtype)
 
 
-def latent_window_attention(q, kc, block_table, seq_lens, qsl, scale: float, window: int, R: int):
+def latent_window_attention(q, kc, block_table, seq_lens, qsl, scale: float, window: int, R: int, sink=None):
     """q [T, H, DK] against the latent rows kc [blocks, bs, DK]: softmax over the keys j <= i with i - j < window
-    (window 0: all of them) of scale * q . row; returns the weighted sums of the rows' first R values, [T, H, R]."""
+    (window 0: all of them) of scale * q . row; returns the weighted sums of the rows' first R values, [T, H, R].
+    ``sink`` fp32 [H]: exp(sink[h]) joins head h's denominator (no key, no value)."""
     T, H, DK = q.shape
     bs = kc.shape[1]
     out = torch.zeros((T, H, R), dtype=torch.float32, device=q.device)
@@ -756,7 +793,8 @@ def latent_window_attention(q, kc, block_table, seq_lens, qsl, scale: float, win
         if window > 0:
             vis = vis & (i - j < window)
         sc = sc.masked_fill(~vis[None], float("-inf"))
-        out[t0:t1] = torch.einsum("hij,jd->ihd", torch.softmax(sc, -1), rows[:, :R])
+        out[t0:t1] = torch.einsum("hij,jd->ihd", softmax_with_sink(sc, sink.view(H, 1, 1) if sink is not None else None),
+                                  rows[:, :R])
     return out.to(q.dtype)
 
 
@@ -833,23 +871,40 @@ def rotate_halves(x, cos, sin, rot: int):
     return torch.cat((u * cos - v * sin, v * cos + u * sin, x[..., rot:].float()), dim=-1)
 
 
+def position_temperature(positions, coef: float, every: int):
+    """fp32 [T]: 1 + coef * ln(floor((p + 1) / every) + 1), the factor queries at position p are multiplied by."""
+    return 1.0 + float(coef) * torch.log((torch.div(positions.long() + 1, int(every), rounding_mode="floor") + 1).float())
+
+
 def qk_norm_rope_cache(qkv, H: int, G: int, D: int, Dv: int, maps: int, q_weight, k_weight, cos_sin, positions,
-                       rot: int, eps: float, k_cache, v_cache, slot_mapping):
+                       rot: int, eps: float, k_cache, v_cache, slot_mapping, pairing: str = "halves", q_temp=None,
+                       v_first=None, v_lam=None):
     """qkv [T, H*maps*D + G*maps*D + G*Dv].  Every D-wide map of every query / key head is divided by its root mean
     square, multiplied by q_weight / k_weight [D] and its first ``rot`` values are rotated (cos_sin fp32 [positions, rot],
-    cosines then sines).  Returns q [T, H, maps * D]; keys go to k_cache [blocks, G, bs, maps * D] and values to v_cache
-    [blocks, G, Dv, bs] at ``slot_mapping``."""
+    cosines then sines; ``pairing``: value i with i + rot / 2, "halves", or 2i with 2i + 1, "neighbours").  ``q_temp`` =
+    (coef, every): queries times ``position_temperature``.  ``v_first`` [T, G * Dv] with ``v_lam`` (one fp32 value):
+    the values become (1 - lam) v + lam v_first before they are cached.  Returns q [T, H, maps * D]; keys go to
+    k_cache [blocks, G, bs, maps * D] and values to v_cache [blocks, G, Dv, bs] at ``slot_mapping``."""
     T = qkv.shape[0]
     nq, nk = H * maps * D, G * maps * D
     q = qkv[:, :nq].float().view(T, H * maps, D)
     k = qkv[:, nq: nq + nk].float().view(T, G * maps, D)
     v = qkv[:, nq + nk:].view(T, G, Dv)
+    if v_first is not None:
+        lam = v_lam.float().reshape(())
+        v = ((1.0 - lam) * v.float() + lam * v_first[:T].float().view(T, G, Dv))
     q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * q_weight.float()
     k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * k_weight.float()
     if rot > 0:
         cs = cos_sin[positions[:T].long()]
         cos, sin = cs[:, None, : rot // 2], cs[:, None, rot // 2: rot]
-        q, k = rotate_halves(q, cos, sin, rot), rotate_halves(k, cos, sin, rot)
+        if pairing == "neighbours":
+            q = torch.cat((rotate_interleaved(q[..., :rot], cos, sin), q[..., rot:]), -1)
+            k = torch.cat((rotate_interleaved(k[..., :rot], cos, sin), k[..., rot:]), -1)
+        else:
+            q, k = rotate_halves(q, cos, sin, rot), rotate_halves(k, cos, sin, rot)
+    if q_temp is not None:
+        q = q * position_temperature(positions[:T], q_temp[0], q_temp[1]).view(T, 1, 1)
     qn = q.to(qkv.dtype).view(T, H, maps * D)
     if k_cache is not None:
         bs = k_cache.shape[2]
@@ -861,14 +916,16 @@ def qk_norm_rope_cache(qkv, H: int, G: int, D: int, Dv: int, maps: int, q_weight
 
 
 def masked_softmax_attention(qn, k_cache, v_cache, block_table, seq_lens, qsl, scale: float, window: int, chunk: int,
-                             sink, maps: int, lam, eps: float, out_scale: float, gate, out_dtype):
+                             sink, maps: int, lam, eps: float, out_scale: float, gate, out_dtype, softcap: float = 0.0,
+                             dist_bias=None):
     """Softmax attention of qn [T, H, maps * D] over the paged keys (k_cache [blocks, G, bs, maps * D], v_cache [blocks,
     G, Dv, bs]); head h reads key / value head h // (H / G).  Key j is visible to the query at position i when j <= i,
     i - j < window (window > 0) and j // chunk == i // chunk (chunk > 0).  ``sink`` fp32 [H]: exp(sink[h]) joins the
     softmax denominator of head h (no key, no value).  maps == 2: each half of a head's row is an attention map of
     its own over the same values, combined as o = a1 - lam * a2 (lam: fp32 tensor of one element), divided by its
     root mean square over Dv and multiplied by out_scale.  ``gate`` [T, H * Dv]: the result is multiplied by its
-    sigmoid.  Returns [T, H * Dv] in ``out_dtype``."""
+    sigmoid.  ``softcap`` > 0: score <- softcap * tanh(score / softcap).  ``dist_bias`` fp32 [far + 1, H]: row
+    min(i - j, far) is added to the (capped) scores of every head.  Returns [T, H * Dv] in ``out_dtype``."""
     T, H, MD = qn.shape
     D = MD // maps
     G, Dv, bs = v_cache.shape[1], v_cache.shape[2], v_cache.shape[3]
@@ -893,6 +950,12 @@ def masked_softmax_attention(qn, k_cache, v_cache, block_table, seq_lens, qsl, s
             vis = vis & (i // chunk == j // chunk)
         q = qn[t0:t1].float().view(L, G, rep, maps, D)
         sc = torch.einsum("igrmd,gjmd->grmij", q, keys.view(G, sl, maps, D)) * scale
+        if softcap > 0:
+            sc = softcap * torch.tanh(sc / softcap)
+        if dist_bias is not None:
+            far = dist_bias.shape[0] - 1
+            b = dist_bias.float()[(i - j).clamp(0, far)]                    # [L, sl, H]
+            sc = sc + b.permute(2, 0, 1).reshape(G, rep, 1, L, sl)
         sc = sc.masked_fill(~vis, float("-inf"))
         mx = sc.max(-1, keepdim=True).values
         if sink is not None:
