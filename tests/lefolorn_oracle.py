@@ -101,7 +101,7 @@ def _mix_values(v, w, m, shared):
         shared["v_first"] = v
         return v
     lam = w["vmix"]
-    return (1 - lam) * v + lam * shared["v_first"]
+    return (1 - lam) * v + lam * shared["v_first"].reshape(v.shape)          # rows of equal width, whatever the heads
 
 
 def _attend(q, k, v, s_fn, ok, extra):
@@ -229,3 +229,130 @@ def forward(cfg, weights, tokens, dtype=torch.float32, want_layers=False):
         trail.append(x)
     logits = group_norm(x, W["final.norm"], groups, eps) @ W["head"].T
     return (logits, torch.stack(trail)) if want_layers else logits
+
+
+# ---- small models ----------------------------------------------------------------------------------------------------
+def feed_forward(ff=40, experts=6, top=2, identity=2, groups=(2, 1), shared=24):
+    r = {"experts": experts, "top": top}
+    if identity:
+        r["identity"] = identity
+    if groups:
+        r["groups"] = {"count": groups[0], "keep": groups[1]}
+    d = {"kind": "moe", "expert": {"ff": ff}, "router": r}
+    if shared:
+        d["shared"] = {"ff": shared}
+    return d
+
+
+def _mlp(mlp):
+    return feed_forward() if mlp == "moe" else mlp
+
+
+def bias_layer(heads=4, kv_heads=2, dim=12, vdim=20, scale=0.3, bias_max=40, q_temp=(0.4, 7), v_mix=False, mlp="moe"):
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale, "bias_max": bias_max}
+    if q_temp:
+        m["q_temp"] = {"coef": q_temp[0], "every": q_temp[1]}
+    if v_mix:
+        m["v_mix"] = True
+    return {"type": "attention", "mixer": m, "mlp": _mlp(mlp)}
+
+
+def cap_layer(heads=4, kv_heads=2, dim=12, vdim=20, window=9, rot_dims=8, base=100.0, scale=0.3, softcap=4.0,
+              v_mix=False, mlp="moe"):
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale}
+    if window:
+        m["mask"] = {"size": window}
+    if rot_dims:
+        m["rot"] = {"base": base, "dims": rot_dims}
+    if softcap:
+        m["softcap"] = softcap
+    if v_mix:
+        m["v_mix"] = True
+    return {"type": "attention_2", "mixer": m, "mlp": _mlp(mlp)}
+
+
+def latent_layer(heads=3, dim=12, rot_dim=8, vdim=20, kv_rank=24, q_rank=16, base=100.0, scale=0.3, mlp="moe"):
+    m = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank, "q_rank": q_rank,
+         "scale": scale, "rot": {"base": base, "dims": rot_dim}}
+    return {"type": "latent_attention", "mixer": m, "mlp": _mlp(mlp)}
+
+
+def make_config(layers, vocab=96, width=48, eps=1e-5, groups=4):
+    return {"architecture": "Lefolorn", "vocab": vocab, "width": width, "norm": {"eps": eps, "groups": groups},
+            "layers": layers}
+
+
+def make_weights(cfg, seed=0, dtype=torch.bfloat16, rows=10):
+    """``rows``: distance buckets of the biased layers (a number, or one per layer index)."""
+    g = torch.Generator().manual_seed(seed)
+    Wd = cfg["width"]
+
+    def lin(o, i, gain=1.0):
+        return torch.randn(o, i, generator=g) * gain / i ** 0.5
+
+    def vec(n, mean=0.0, spread=0.1):
+        return mean + spread * torch.randn(n, generator=g)
+    W = {"embed": torch.randn(cfg["vocab"], Wd, generator=g), "final.norm": vec(Wd, 1.0),
+         "head": lin(cfg["vocab"], Wd, 2.0)}
+    for i, spec in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", spec["mixer"]
+        W[p + "norm1"] = vec(Wd, 1.0, 0.2)
+        W[p + "ls1"], W[p + "ls2"] = vec(Wd, 0.8, 0.3), vec(Wd, 0.8, 0.3)
+        for n in ("rg1", "rg2"):
+            W[p + n], W[p + n + ".b"] = lin(Wd, Wd, 2.0), vec(Wd, 0.5, 0.5)
+        H, E = m["heads"], m["vdim"]
+        if spec["type"] == "latent_attention":
+            D, P, R, Q = m["dim"], m["rot_dim"], m["kv_rank"], m["q_rank"]
+            W[p + "mix.dq"], W[p + "mix.dq.norm"] = lin(Q, Wd, 2.0), vec(Q, 1.0, 0.2)
+            W[p + "mix.uq"] = lin(H * (D + P), Q, 2.0)
+            W[p + "mix.dkv"], W[p + "mix.dkv.norm"] = lin(R + P, Wd, 2.0), vec(R, 1.0, 0.2)
+            W[p + "mix.uk"], W[p + "mix.uv"] = lin(H * D, R, 2.0), lin(H * E, R)
+            W[p + "mix.sink"] = vec(H, 0.5, 1.0)
+        else:
+            G, D = m["kv_heads"], m["dim"]
+            for n, r_ in (("q", H * D), ("k", G * D), ("v", G * E)):
+                W[p + "mix." + n] = lin(r_, Wd, 2.0)
+                W[p + "mix." + n + ".b"] = vec(r_, 0.0, 0.3)
+            W[p + "mix.q.norm"], W[p + "mix.k.norm"] = vec(D, 1.0, 0.2), vec(D, 1.0, 0.2)
+            if m.get("v_mix"):
+                W[p + "mix.vmix"] = vec((), 0.4, 0.2)
+            if spec["type"] == "attention":
+                n_rows = rows[i] if isinstance(rows, dict) else rows
+                W[p + "mix.rel"] = torch.randn(n_rows, H, generator=g) * 1.5
+                W[p + "mix.g"] = lin(H * E, Wd, 2.0)
+        W[p + "mix.o"] = lin(Wd, H * E)
+        mlp = spec.get("mlp")
+        if mlp is None:
+            del W[p + "ls2"], W[p + "rg2"], W[p + "rg2.b"]
+            continue
+        r = mlp["router"]
+        n = r["experts"] + r.get("identity", 0)
+        W[p + "mlp.router"] = lin(n, Wd, 3.0)
+        W[p + "mlp.correction"] = vec(n, -0.1, 0.15)                         # choice scores of both signs
+        for e in range(r["experts"]):
+            W[p + f"mlp.e{e}.gate"] = lin(mlp["expert"]["ff"], Wd, 1.5)
+            W[p + f"mlp.e{e}.up"] = lin(mlp["expert"]["ff"], Wd, 1.5)
+            W[p + f"mlp.e{e}.down"] = lin(Wd, mlp["expert"]["ff"])
+        if mlp.get("shared"):
+            W[p + "mlp.shared.gate"] = lin(mlp["shared"]["ff"], Wd, 1.5)
+            W[p + "mlp.shared.up"] = lin(mlp["shared"]["ff"], Wd, 1.5)
+            W[p + "mlp.shared.down"] = lin(Wd, mlp["shared"]["ff"])
+    return {k: v.to(dtype) for k, v in W.items()}
+
+
+def save_checkpoint(folder, cfg, W):
+    from safetensors.torch import save_file
+    os.makedirs(folder, exist_ok=True)
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    save_file({k: v.contiguous() for k, v in W.items()}, os.path.join(folder, "model.safetensors"))
+    return folder
+
+
+def logit_error(got, want):
+    """Root mean square of the difference (its mean over the vocabulary taken off), relative to the spread of the
+    wanted logits."""
+    d = got.float() - want.float()
+    d = d - d.mean(-1, keepdim=True)
+    spread = (want.float() - want.float().mean(-1, keepdim=True)).pow(2).mean().sqrt()
+    return (d.pow(2).mean().sqrt() / spread).item()

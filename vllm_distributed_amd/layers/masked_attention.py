@@ -180,7 +180,7 @@ class MaskedSoftmaxAttention(nn.Module):
         # score map a key head of its own in the cache); anything else, fp32 included: the kernel for any sizes
         self.use_mfma = ops.masked_attention_mfma_ok(H, G, D, Dv, maps, self.sink is not None, cfg.model_config.dtype,
                                                      cfg.device_config.device != "cpu") \
-            and cfg.cache_config.cache_dtype == "auto" and not self.dist_far
+            and cfg.cache_config.cache_dtype == "auto" and not (self.dist_far and maps == 2)
         self.max_len = int(cfg.model_config.max_model_len) + 1
         self._cos_sin: Optional[torch.Tensor] = None
 

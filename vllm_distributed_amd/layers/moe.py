@@ -63,6 +63,28 @@ def grouped_topk(scores: torch.Tensor, k: int, renormalize: bool, num_expert_gro
     return w.float(), ids.to(torch.int32)
 
 
+def grouped_topk_with_identity(logits: torch.Tensor, bias: Optional[torch.Tensor], k: int, groups: int, keep: int,
+                               renormalize: bool, scoring: str = "softmax", group_score: str = "max",
+                               identity: int = 0, renorm_eps: float = 0.0):
+    """Group-limited choice over router outputs whose last ``identity`` have no expert behind them (such an "expert"
+    returns its input): one launch on the device, PyTorch ops elsewhere.  Returns (weights f32 [T, k], ids i32 [T, k],
+    identity weights f32 [T] or None); identity winners come back as id -1 with weight 0 and their weights' sum per
+    token in the third result."""
+    routed = ops.moe_grouped_topk(logits, bias, k, groups, keep, renormalize, scoring, group_score, identity,
+                                  renorm_eps)
+    if routed is not None:
+        return routed
+    scores = torch.softmax(logits.float(), -1) if scoring == "softmax" else torch.sigmoid(logits.float())
+    w, ids = grouped_topk(scores, k, renormalize, groups, keep, bias, group_score, renorm_eps)
+    idw = None
+    if identity:
+        ident = ids >= logits.shape[1] - identity
+        idw = (w * ident).sum(-1)
+        w = w.masked_fill(ident, 0.0)
+        ids = ids.masked_fill(ident, -1)
+    return w, ids, idw
+
+
 class UnquantizedMoEMethod:
     def create_weights(self, layer: "FusedMoE", E: int, H: int, I: int, dtype: torch.dtype) -> None:
         w13 = nn.Parameter(torch.empty(E, (2 if getattr(layer, "gated", True) else 1) * I, H, dtype=dtype),
@@ -247,26 +269,12 @@ class FusedMoE(nn.Module):
         return ops.moe_topk_softmax(router_logits, k, self.renormalize)
 
     def _select_grouped(self, router_logits: torch.Tensor):
-        """Group-limited choice with every option (scoring, group score, identity outputs, renormalisation constant):
-        one launch on the device, PyTorch ops elsewhere.  Identity winners come back as id -1 / weight 0; their
-        weights' sum per token lands in ``identity_weight``."""
-        k, E = self.top_k, self.global_num_experts
+        """Group-limited choice with every option (scoring, group score, identity outputs, renormalisation constant);
+        the weights identity outputs won land in ``identity_weight``."""
         top2 = (self.e_score_correction_bias is not None) if self.group_score is None else self.group_score == "top2"
-        routed = ops.moe_grouped_topk(router_logits, self.e_score_correction_bias, k, self.num_expert_group,
-                                      self.topk_group, self.renormalize, self.scoring_func,
-                                      "top2" if top2 else "max", self.num_identity, self.renorm_eps)
-        if routed is not None:
-            w, ids, self.identity_weight = routed
-            return w, ids
-        scores = torch.softmax(router_logits.float(), -1) if self.scoring_func == "softmax" \
-            else torch.sigmoid(router_logits.float())
-        w, ids = grouped_topk(scores, k, self.renormalize, self.num_expert_group, self.topk_group,
-                              self.e_score_correction_bias, "top2" if top2 else "max", self.renorm_eps)
-        if self.num_identity:
-            ident = ids >= E
-            self.identity_weight = (w * ident).sum(-1)
-            w = w.masked_fill(ident, 0.0)
-            ids = ids.masked_fill(ident, -1)
+        w, ids, self.identity_weight = grouped_topk_with_identity(
+            router_logits, self.e_score_correction_bias, self.top_k, self.num_expert_group, self.topk_group,
+            self.renormalize, self.scoring_func, "top2" if top2 else "max", self.num_identity, self.renorm_eps)
         return w, ids
 
     def _forward_ep_dispatch(self, x: torch.Tensor, lg: torch.Tensor, routed=None) -> torch.Tensor:

@@ -245,14 +245,15 @@ def paged_attention_decode(out, q, k_cache, v_cache, block_table, seq_lens, q_st
                            num_splits: int = 1, max_q_len: int = 1, window: int = 0, softcap: float = 0.0,
                            alibi: Optional[torch.Tensor] = None, workspace=None, k_scale: float = 1.0,
                            v_scale: float = 1.0, sink: Optional[torch.Tensor] = None, chunk: int = 0,
-                           v_shift: int = 0):
+                           v_shift: int = 0, dist_bias: Optional[torch.Tensor] = None):
     """q, out: [T, Hq, D].  Each sequence has <= max_q_len query tokens (1 for plain decode).
     ``sink`` fp32 [Hq]: exp(sink[h]) joins head h's softmax denominator; ``chunk`` > 0: keys of the query's own chunk
-    of that many positions only; ``v_shift``: K head k reads V head k >> v_shift (v_cache holds that many fewer heads).
-    These three are options of the device kernels only."""
+    of that many positions only; ``v_shift``: K head k reads V head k >> v_shift (v_cache holds that many fewer heads);
+    ``dist_bias`` fp32 [far + 1, Hq]: row min(query position - key position, far) joins the scores.
+    These four are options of the device kernels only."""
     T, Hq, D = q.shape
     if not _dev(q):
-        assert sink is None and not chunk and not v_shift
+        assert sink is None and not chunk and not v_shift and dist_bias is None
         out.copy_(R.paged_attention(q, k_cache, v_cache, block_table, seq_lens, q_start_loc, scale, window,
                                     softcap, alibi, k_scale=k_scale, v_scale=v_scale))
         return out
@@ -268,15 +269,23 @@ def paged_attention_decode(out, q, k_cache, v_cache, block_table, seq_lens, q_st
            block_table.data_ptr(), seq_lens.data_ptr(), q_start_loc.data_ptr(), N.ptr(alibi), N.ptr(part_out),
            N.ptr(part_lse), S, T, Hq, k_cache.shape[1], D, k_cache.shape[2], block_table.stride(0), num_splits,
            max_q_len, q.stride(0), out.stride(0), scale, softcap, window, N.dt(q.dtype), _kv_fp8(k_cache), k_scale,
-           v_scale, N.ptr(sink), int(chunk), int(v_shift), N.stream())
+           v_scale, N.ptr(sink), int(chunk), int(v_shift), *_dist_bias_args(dist_bias, Hq), N.stream())
     return out
+
+
+def _dist_bias_args(dist_bias: Optional[torch.Tensor], Hq: int) -> tuple:
+    if dist_bias is None:
+        return None, 0
+    assert dist_bias.dtype == torch.float32 and dist_bias.is_contiguous() and dist_bias.dim() == 2 \
+        and dist_bias.shape[1] == Hq
+    return dist_bias.data_ptr(), dist_bias.shape[0] - 1
 
 
 def paged_attention_prefill(out, q, k_cache, v_cache, block_table, seq_lens, q_start_loc, scale: float,
                             window: int = 0, softcap: float = 0.0, alibi: Optional[torch.Tensor] = None,
                             k_scale: float = 1.0, v_scale: float = 1.0, causal: bool = True,
                             return_lse: bool = False, max_q_len: int = 0, sink: Optional[torch.Tensor] = None,
-                            chunk: int = 0, v_shift: int = 0):
+                            chunk: int = 0, v_shift: int = 0, dist_bias: Optional[torch.Tensor] = None):
     """Varlen attention of new tokens against the paged cache.  ``causal=False``: every query token sees
     all ``seq_lens[s]`` keys of its sequence (encoder models, the shared-prefix pass of cascade
     attention).  ``return_lse``: also return the log-sum-exp [Hq, T] (natural log) of every row.
@@ -284,7 +293,8 @@ def paged_attention_prefill(out, q, k_cache, v_cache, block_table, seq_lens, q_s
     the wide kernel then starts the longest causal tiles of all sequences first."""
     T, Hq, D = q.shape
     if not _dev(q):
-        assert sink is None and not chunk and not v_shift        # options of the device kernels (see the decode form)
+        # options of the device kernels (see the decode form)
+        assert sink is None and not chunk and not v_shift and dist_bias is None
         o, lse = R.paged_attention(q, k_cache, v_cache, block_table, seq_lens, q_start_loc, scale, window,
                                    softcap, alibi, return_lse=True, k_scale=k_scale, v_scale=v_scale,
                                    causal=causal)
@@ -295,7 +305,7 @@ def paged_attention_prefill(out, q, k_cache, v_cache, block_table, seq_lens, q_s
            block_table.data_ptr(), seq_lens.data_ptr(), q_start_loc.data_ptr(), N.ptr(alibi), seq_lens.shape[0], T,
            Hq, k_cache.shape[1], D, k_cache.shape[2], block_table.stride(0), q.stride(0), out.stride(0), scale,
            softcap, window, N.dt(q.dtype), _kv_fp8(k_cache), k_scale, v_scale, int(bool(causal)), N.ptr(lse),
-           int(max_q_len), N.ptr(sink), int(chunk), int(v_shift), N.stream())
+           int(max_q_len), N.ptr(sink), int(chunk), int(v_shift), *_dist_bias_args(dist_bias, Hq), N.stream())
     return (out, lse) if return_lse else out
 
 
@@ -1772,9 +1782,8 @@ def masked_softmax_attention_mfma(qn: torch.Tensor, k_cache: torch.Tensor, v_cac
     a = torch.empty((T, Hq, D), dtype=qn.dtype, device=qn.device)
     nd, ndt, n_pre = int(num_decode_seqs), int(num_decode_tokens), int(num_prefill_seqs)
     R_ = H // G
-    if dist_bias is not None:
-        raise NotImplementedError("a distance bias table on the matrix-core attention path")
-    kw = dict(window=int(window), sink=sink, chunk=int(chunk), v_shift=maps - 1, softcap=float(softcap))
+    kw = dict(window=int(window), sink=sink, chunk=int(chunk), v_shift=maps - 1, softcap=float(softcap),
+              dist_bias=dist_bias)
     cols = max(int(max_decode_query_len), 1) * R_
     if nd > 0 and (cols > 32 or (cols > 16 and D > 128)):
         raise ValueError(f"{cols} query columns per key head and step are beyond the decode form")

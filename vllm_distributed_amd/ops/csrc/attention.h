@@ -32,6 +32,8 @@ struct AttnParams {
   const float* sink;        // [Hq]: exp(sink[h]) joins head h's softmax denominator, with no key and no value
   int chunk;                // > 0: the query at position i sees keys j with j / chunk == i / chunk only
   int v_shift;              // K head k reads V head k >> v_shift (the V cache then holds Hkv >> v_shift heads)
+  const float* dist_bias;   // [dist_far + 1, Hq]: row min(query position - key position, dist_far) joins the scores
+  int dist_far;             //   of every head (after the scale and the soft cap)
 };
 
 // Key selection of the sparse prefill form: per (sequence, head) a list of single key positions ("vertical" lines of

@@ -64,7 +64,8 @@ __global__ __launch_bounds__(256) void paged_attn_kernel(AttnParams p) {
   // column c of the workgroup -> (query token c / G, head c % G)
   int limit[NCT], lower[NCT];
   long col_off[NCT];           // element offset of (token, head) in q / out
-  float slope[NCT], sink_m[NCT];
+  float slope[NCT], sink_m[NCT], bfar2[NCT];
+  const float* bias_col[NCT];
   V8 qf[NCT][KS];
   int wave_hi = 0, wave_lo = 0x7fffffff;
 #pragma unroll
@@ -79,6 +80,8 @@ __global__ __launch_bounds__(256) void paged_attn_kernel(AttnParams p) {
     if (valid && p.chunk > 0) lower[ct] = max(lower[ct], (limit[ct] - 1) / p.chunk * p.chunk);
     const int head = kvh * G + h;
     slope[ct] = (p.alibi && valid) ? p.alibi[head] : 0.f;
+    bias_col[ct] = p.dist_bias ? p.dist_bias + head : nullptr;
+    bfar2[ct] = (p.dist_bias && valid) ? p.dist_bias[(long)p.dist_far * p.Hq + head] * 1.4426950408889634f : 0.f;
     // a sink is a score without key or value: the running maximum starts there and the sum with its weight of one
     // (once per column: in the lane group that holds the sum's first part, and in split mode in one wave of one part)
     sink_m[ct] = (p.sink && valid && (!SPLIT || (wave == 0 && blockIdx.z == 0))) ? p.sink[head] * 1.4426950408889634f
@@ -169,6 +172,7 @@ __global__ __launch_bounds__(256) void paged_attn_kernel(AttnParams p) {
         float x = sv[j] * p.scale;
         if (p.softcap > 0.f) x = p.softcap * tanhf(x / p.softcap);
         x += slope[ct] * (float)(tok - (limit[ct] - 1));
+        if (p.dist_bias) x += bias_col[ct][(long)min(max(limit[ct] - 1 - tok, 0), p.dist_far) * p.Hq];
         x *= 1.4426950408889634f;
         x = (tok < limit[ct] && tok >= lower[ct]) ? x : -INFINITY;
         sv[j] = x;
@@ -358,7 +362,8 @@ __global__ __launch_bounds__(256, PREFILL_WGS_PER_CU) void paged_prefill_lds_ker
 
   int limit[NCT], lower[NCT];
   long col_off[NCT];
-  float slope[NCT], sink_m[NCT];
+  float slope[NCT], sink_m[NCT], bfar2[NCT];
+  const float* bias_col[NCT];
   V8 qf[NCT][KS];
   int wave_hi = 0, wave_lo = 0x7fffffff;
 #pragma unroll
@@ -372,6 +377,8 @@ __global__ __launch_bounds__(256, PREFILL_WGS_PER_CU) void paged_prefill_lds_ker
     if (valid && p.chunk > 0) lower[ct] = max(lower[ct], (limit[ct] - 1) / p.chunk * p.chunk);
     const int head = head0 + h;
     slope[ct] = (p.alibi && valid) ? p.alibi[head] : 0.f;
+    bias_col[ct] = p.dist_bias ? p.dist_bias + head : nullptr;
+    bfar2[ct] = (p.dist_bias && valid) ? p.dist_bias[(long)p.dist_far * p.Hq + head] * 1.4426950408889634f : 0.f;
     sink_m[ct] = (p.sink && valid) ? p.sink[head] * 1.4426950408889634f : -INFINITY;
     const T* qp = (const T*)p.q + (long)(qs + (valid ? qt : q0)) * p.q_stride + (long)head * D + g * DQ;
 #pragma unroll
@@ -500,7 +507,8 @@ __global__ __launch_bounds__(256, PREFILL_WGS_PER_CU) void paged_prefill_lds_ker
   auto compute = [&](int step, int buf) {
     const int tb0 = step * 32;
     if (!(tb0 < wave_hi && tb0 + 32 > wave_lo)) return;   // wave-uniform: tile outside this wave's causal range
-    const bool fast = plain && tb0 + 32 <= full_hi && tb0 >= full_lo;
+    const bool far_tile = p.dist_bias != nullptr && tb0 + 32 <= full_hi - p.dist_far;
+    const bool fast = plain && tb0 + 32 <= full_hi && tb0 >= full_lo && (p.dist_bias == nullptr || far_tile);
     V8 kf[2][KS], vf[NT];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
@@ -529,7 +537,7 @@ __global__ __launch_bounds__(256, PREFILL_WGS_PER_CU) void paged_prefill_lds_ker
         // feeds the exponential, so a score costs max + fma + exp + add
 #pragma unroll
         for (int j = 0; j < 8; ++j) mx = fmaxf(mx, sv[j]);
-        mx *= sl2;
+        mx = fmaf(mx, sl2, bfar2[ct]);
       } else {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
@@ -538,6 +546,10 @@ __global__ __launch_bounds__(256, PREFILL_WGS_PER_CU) void paged_prefill_lds_ker
           if (p.softcap > 0.f) x = p.softcap * tanhf(x / p.softcap);
           x += slope[ct] * (float)(tok - (limit[ct] - 1));
           x *= 1.4426950408889634f;
+          // a tile at least dist_far behind every column of the wave takes the table's last row throughout
+          if (p.dist_bias)
+            x += far_tile ? bfar2[ct] : 1.4426950408889634f *
+                 bias_col[ct][(long)min(max(limit[ct] - 1 - tok, 0), p.dist_far) * p.Hq];
           x = (tok < limit[ct] && tok >= lower[ct]) ? x : -INFINITY;
           sv[j] = x;
           mx = fmaxf(mx, x);
@@ -552,9 +564,10 @@ __global__ __launch_bounds__(256, PREFILL_WGS_PER_CU) void paged_prefill_lds_ker
       float ps = 0.f;
       V8 pb;
       const float mul = fast ? sl2 : 1.f;
+      const float off = (fast ? bfar2[ct] : 0.f) - m_use;
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const float e = fexp2(fmaf(sv[j], mul, -m_use));
+        const float e = fexp2(fmaf(sv[j], mul, off));
         ps += e;
         pb[j] = (T)e;
       }
@@ -780,16 +793,17 @@ VDA_EXPORT int vda_paged_attention_decode(
     const int* seq_lens, const int* q_start_loc, const float* alibi, float* part_out, float* part_lse,
     int num_seqs, int num_tokens, int Hq, int Hkv, int D, int block_size, int max_blocks, int nsplit,
     int max_q_len, long q_stride, long out_stride, float scale, float softcap, int window, int dtype,
-    int kv_fp8, float k_scale, float v_scale, const float* sink, int chunk, int v_shift, hipStream_t st) {
+    int kv_fp8, float k_scale, float v_scale, const float* sink, int chunk, int v_shift, const float* dist_bias,
+    int dist_far, hipStream_t st) {
   if (Hq % Hkv) return -1;
-  if (chunk < 0 || v_shift < 0 || (Hkv >> v_shift) << v_shift != Hkv) return -7;
+  if (chunk < 0 || v_shift < 0 || (Hkv >> v_shift) << v_shift != Hkv || (dist_bias && dist_far < 0)) return -7;
   if (nsplit < 1 || nsplit > 64) return -6;      // the reduce kernel keeps one partition per lane
   const int cols = max_q_len * (Hq / Hkv);
   if (cols > 32 || (cols > 16 && D > 128)) return -4;
   AttnParams p{q, k_cache, v_cache, out, part_out, part_lse, block_table, seq_lens, q_start_loc, alibi,
                num_seqs, Hq, Hkv, max_blocks, nsplit, q_stride, out_stride, scale * (kv_fp8 ? k_scale : 1.f), softcap,
                kv_fp8 ? v_scale : 1.f, window, 0, 1, num_tokens, nullptr};
-  p.sink = sink; p.chunk = chunk; p.v_shift = v_shift;
+  p.sink = sink; p.chunk = chunk; p.v_shift = v_shift; p.dist_bias = dist_bias; p.dist_far = dist_far;
   const int form = cols <= 16 ? 0 : 1;
   int rc = dtype == VDA_BF16 ? dispatch_d<bf16_t>(p, D, block_size, form, num_seqs, st, kv_fp8)
                              : dispatch_d<f16_t>(p, D, block_size, form, num_seqs, st, kv_fp8);
@@ -829,18 +843,20 @@ VDA_EXPORT int vda_paged_attention_prefill(
     const int* seq_lens, const int* q_start_loc, const float* alibi, int num_seqs, int num_tokens,
     int Hq, int Hkv, int D, int block_size, int max_blocks, long q_stride, long out_stride, float scale,
     float softcap, int window, int dtype, int kv_fp8, float k_scale, float v_scale, int causal, float* lse_out,
-    int max_q_len, const float* sink, int chunk, int v_shift, hipStream_t st) {
+    int max_q_len, const float* sink, int chunk, int v_shift, const float* dist_bias, int dist_far, hipStream_t st) {
   if (Hq % Hkv) return -1;
   const int G = Hq / Hkv;
   if (G > 128) return -4;
   if (!causal && (window > 0 || chunk > 0)) return -5;
   if (chunk < 0 || v_shift < 0 || (Hkv >> v_shift) << v_shift != Hkv) return -7;
-  const bool extras = sink != nullptr || chunk > 0 || v_shift > 0;     // not in the direct-to-register form
+  if (dist_bias && dist_far < 0) return -7;
+  // not in the direct-to-register form
+  const bool extras = sink != nullptr || chunk > 0 || v_shift > 0 || dist_bias != nullptr;
   const int q_tile = 128 / G;     // 4 waves x 32 columns
   AttnParams p{q, k_cache, v_cache, out, nullptr, nullptr, block_table, seq_lens, q_start_loc, alibi,
                num_seqs, Hq, Hkv, max_blocks, 1, q_stride, out_stride, scale * (kv_fp8 ? k_scale : 1.f), softcap,
                kv_fp8 ? v_scale : 1.f, window, q_tile, causal, num_tokens, lse_out, max_q_len};
-  p.sink = sink; p.chunk = chunk; p.v_shift = v_shift;
+  p.sink = sink; p.chunk = chunk; p.v_shift = v_shift; p.dist_bias = dist_bias; p.dist_far = dist_far;
   // Wide form (8 waves, 256 columns, 64-key tiles): head size 128 and enough query tiles to occupy the
   // chip (one workgroup per CU); short chunks keep the 4-wave form, which cuts them into more workgroups.
   if (D == 128 && 256 % G == 0 && (g_prefill_variant == 1 || g_prefill_variant == 3)) {

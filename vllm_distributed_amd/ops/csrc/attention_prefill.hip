@@ -126,6 +126,7 @@ __global__ __launch_bounds__(512) void paged_prefill_wide_kernel(AttnParams p, i
   int lower = (valid && p.window > 0) ? max(0, limit - p.window) : 0;
   if (valid && p.chunk > 0) lower = max(lower, (limit - 1) / p.chunk * p.chunk);     // keys of the query's chunk only
   const float slope = (p.alibi && valid) ? p.alibi[head] : 0.f;
+  const float* bias_col = p.dist_bias ? p.dist_bias + head : nullptr;      // this column's distance biases
   const long col_off = valid ? (long)(qs + qt) : -1;
   V8 qf[8];
   {
@@ -227,7 +228,7 @@ __global__ __launch_bounds__(512) void paged_prefill_wide_kernel(AttnParams p, i
   // vector ALU and the matrix pipe have independent work inside one wave:
   //     scores(0) . scores(1) || softmax(0) . rescale . P.V(0) || softmax(1) . rescale . P.V(1)
   // (a || b: same basic block, no dependence).  MODE 0: no masking, scale folded into the exponent's fma;
-  // 1: causal / window masking only; 2: soft-cap and ALiBi as well (its own kernel instance, GENERAL, so
+  // 1: causal / window masking only; 2: soft-cap, ALiBi and a distance-bias table as well (its own kernel instance, GENERAL, so
   // that the common instance does not pay for its registers).
   f32x16 S[2];
   auto qk_half = [&](int buf, int kb) {
@@ -252,6 +253,7 @@ __global__ __launch_bounds__(512) void paged_prefill_wide_kernel(AttnParams p, i
           x *= p.scale;
           if (p.softcap > 0.f) x = p.softcap * tanhf(x / p.softcap);
           x += slope * (float)(tok - (limit - 1));
+          if (bias_col) x += bias_col[(long)min(max(limit - 1 - tok, 0), p.dist_far) * p.Hq];
           x *= 1.4426950408889634f;
         }
         x = (tok < limit && tok >= lower) ? x : -INFINITY;
@@ -424,7 +426,7 @@ int launch_bs(const AttnParams& p, int bs, int ntiles, hipStream_t st) {
 
 template <typename T, bool F8>
 int launch_mode(const AttnParams& p, int bs, int ntiles, hipStream_t st) {
-  const bool general = p.softcap > 0.f || p.alibi != nullptr;
+  const bool general = p.softcap > 0.f || p.alibi != nullptr || p.dist_bias != nullptr;
   return general ? launch_bs<T, F8, true>(p, bs, ntiles, st) : launch_bs<T, F8, false>(p, bs, ntiles, st);
 }
 
