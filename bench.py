@@ -149,6 +149,10 @@ def main() -> None:
     ap.add_argument("--compare-sevazen", action="store_true",
                     help="likewise for Sevazen stacks (window attention with sinks, differential attention in chunks, "
                          "routed squared-ReLU experts) beside a sliding-window Mixtral stack of equal size")
+    ap.add_argument("--compare-lefolorn", action="store_true",
+                    help="likewise for Lefolorn stacks (latent attention with sinks, distance-bias attention, soft-capped "
+                         "window attention, parallel gated sub-layers, routed experts with identity outputs) beside a "
+                         "Sevazen and a sliding-window Mixtral stack of equal size")
     ap.add_argument("--sizes", default="small,medium", help="--compare-...: small, medium, large")
     ap.add_argument("--rehearse-on-one-gpu", action="store_true", help="--disagg: every engine on GPU 0")
     ap.add_argument("--kv-push", action="store_true", help="--disagg: push blocks while prefilling (landing pool)")
@@ -157,10 +161,11 @@ def main() -> None:
     a = ap.parse_args()
     if a.disagg:
         return run_disagg(a)
-    if a.compare_nositar or a.compare_rapovik or a.compare_sevazen:
+    if a.compare_nositar or a.compare_rapovik or a.compare_sevazen or a.compare_lefolorn:
         from vllm_distributed_amd.benchmarks import hybrid_compare
         argv = (["--models", "rapovik,jamba-moe"] if a.compare_rapovik else
-                ["--models", "sevazen,mixtral-swa"] if a.compare_sevazen else []) + ["--sizes", a.sizes, "--batch", str(32 if a.batch == 256 else a.batch),
+                ["--models", "sevazen,mixtral-swa"] if a.compare_sevazen else
+                ["--models", "lefolorn,sevazen,mixtral-swa"] if a.compare_lefolorn else []) + ["--sizes", a.sizes, "--batch", str(32 if a.batch == 256 else a.batch),
                 "--input-len", str(2048 if a.input_len == 1024 else a.input_len),
                 "--output-len", str(64 if a.output_len == 128 else a.output_len)]
         hybrid_compare.main(argv + (["--enforce-eager"] if a.enforce_eager else []))

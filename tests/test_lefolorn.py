@@ -144,7 +144,10 @@ def test_gated_parallel_residual_with_group_norm(dev, dt, W_, groups):
             ([(y1, s1, g1, None, None), (y2, s2, g2, h, idw)],
              x + (y1.float() * s1 * torch.sigmoid(g1.float())
                   + (y2.float() + idw[:, None] * h.float()) * s2 * torch.sigmoid(g2.float()))),
-            ([(y1, None, None, None, None), (y2, s2, None, None, None)], x + (y1.float() + y2.float() * s2))):
+            ([(y1, None, None, None, None), (y2, s2, None, None, None)], x + (y1.float() + y2.float() * s2)),
+            ([(y1, s1, g1, None, None), (y2, s2, g2, h, idw), (g1, s2, g2, None, None)],
+             x + (y1.float() * s1 * torch.sigmoid(g1.float())
+                  + (y2.float() + idw[:, None] * h.float() + g1.float()) * s2 * torch.sigmoid(g2.float())))):
         xd = x.clone().to(dev)
         nxt = ops.gated_residual_group_norm(xd, [tuple(d(t) for t in sub) for sub in subs], d(w), groups, eps, dt)
         torch.testing.assert_close(xd.cpu(), want, atol=3e-5, rtol=1e-5)
@@ -243,8 +246,21 @@ def test_attention_paged(dev, dt, H, G, D, E, kind, window, cap, dist, temp, rot
     starts inside a page, a whole prompt -- against the oracle's dense computation per sequence; contexts longer than
     windows and bias tables, so that hidden and far keys sit in pages of their own.  The bias table's rows differ by
     O(1), so a key in the wrong bucket shows."""
+    paged_case(dev, dt, H, G, D, E, kind, window, cap, dist, temp, rot, vmix, bs, [75, 53, 20], [1, 11, 20])
+
+
+@pytest.mark.parametrize("dev,dt", OP_CASES)
+@pytest.mark.parametrize("H,G,D,E,kind,window,cap,dist,temp,rot,vmix", [
+    (4, 2, 64, 64, "bias", 0, 0.0, (16, 40), (0.3, 100), 0, False), (2, 1, 128, 128, "bias", 0, 0.0, (12, 70), None, 0, True),
+    (4, 1, 128, 128, "cap", 150, 8.0, None, None, 32, False), (3, 1, 16, 24, "bias", 0, 0.0, (6, 100), None, 0, False)])
+def test_attention_paged_long(dev, dt, H, G, D, E, kind, window, cap, dist, temp, rot, vmix):
+    """Hundreds of keys: whole key tiles lie beyond the bias table's end (they take its last row as a constant) or
+    outside the window, next to tiles that straddle those edges."""
+    paged_case(dev, dt, H, G, D, E, kind, window, cap, dist, temp, rot, vmix, 16, [330, 290, 300], [1, 130, 300])
+
+
+def paged_case(dev, dt, H, G, D, E, kind, window, cap, dist, temp, rot, vmix, bs, lens, news):
     eps, scale, lam_v = 1e-5, 0.35, 0.3
-    lens, news = [75, 53, 20], [1, 11, 20]
     nq, nk, nv = H * D, G * D, G * E
     ng = H * E if kind == "bias" else 0
     cols = nq + nk + nv + ng
@@ -272,7 +288,7 @@ def test_attention_paged(dev, dt, H, G, D, E, kind, window, cap, dist, temp, rot
     cs = None
     if rot:
         from vllm_distributed_amd.layers.latent_attention import interleaved_cos_sin
-        cs = interleaved_cos_sin(128, rot, 40.0, torch.device(dev))
+        cs = interleaved_cos_sin(512, rot, 40.0, torch.device(dev))
     sink = torch.zeros(H, device=dev) if kind == "bias" else None
     bias = None
     if dist:
@@ -303,7 +319,8 @@ def test_attention_paged(dev, dt, H, G, D, E, kind, window, cap, dist, temp, rot
         def run(splits):
             return ops.masked_softmax_attention_mfma(qn, kc, vc, table.to(dev), sl, qsl, qsl[1:] - 1, 1, 1, 2,
                                                      sum(news[1:]), 1, splits, max(news), scale, H, window, 0, sink,
-                                                     1, None, eps, 1.0, gt, softcap=cap, dist_bias=bias)
+                                                     1, None, eps, 1.0, gt, softcap=cap,
+                                                     dist_bias=ops.padded_distance_rows(bias) if dist else None)
         got = run(1)
         assert rel(run(3), got) < 1e-2
         if D == 128:                                  # the 8-wave form for prompts, whenever the shape allows

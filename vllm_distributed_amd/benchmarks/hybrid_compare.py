@@ -1,9 +1,10 @@
-"""Prefill and decode throughput of a Nositar, Rapovik or Sevazen stack beside the closest existing models of equal size, random
-weights.
+"""Prefill and decode throughput of a Nositar, Rapovik, Sevazen or Lefolorn stack beside the closest existing models of
+equal size, random weights.
 
     python bench.py --compare-nositar [--sizes small,medium] [--batch 32] [--input-len 2048] [--output-len 64]
     python bench.py --compare-rapovik [...]        (rapovik beside jamba-moe)
     python bench.py --compare-sevazen [...]        (sevazen beside mixtral-swa)
+    python bench.py --compare-lefolorn [...]       (lefolorn beside sevazen and mixtral-swa)
 
 Per size three engines run one after the other, each in a process of its own (``--one`` is the child's entry):
   nositar      alternating sigmoid head-mixing attention (window + kept first tokens) and gated delta-rule layers,
@@ -17,6 +18,10 @@ Per size three engines run one after the other, each in a process of its own (``
   sevazen      window attention with sinks and a short convolution and differential attention inside chunks in turn,
                fp32 residual with layer norms on the sub-layers' outputs, 8 routed squared-ReLU experts (two per token)
                plus a shared expert in every layer
+  lefolorn     latent attention with sinks, distance-bias attention with an output gate and soft-capped window attention
+               in turn; both sub-layers of a layer read one group norm of the fp32 residual and join it behind layer
+               scales and per-channel sigmoid gates; every layer has 8 routed gated experts and 2 identity outputs (two
+               choices per token, from the better of two groups) plus a shared expert
   mixtral-swa  a Mixtral stack of the same width, depth and heads with the same sliding window and 8 routed gated
                experts (two per token) of equal weight count
 Prefill: ``batch`` prompts of ``input-len`` tokens, one generated token.  Decode: the same requests generating
@@ -128,7 +133,29 @@ def sevazen_config(s: dict) -> dict:
             "layers": [dict(win if i % 2 == 0 else dif, mlp=moe) for i in range(s["layers"])]}
 
 
-MODELS = {"sevazen": sevazen_config, "mixtral-swa": mixtral_swa_config, "nositar": nositar_config, "llama-swa": llama_config, "jamba": jamba_config, "jamba-moe": jamba_moe_config,
+def lefolorn_config(s: dict) -> dict:
+    """Latent attention (sinks; latent of 128 + 32 for heads of 64, 512 + 64 for heads of 128: the sizes the
+    matrix-core latent kernel has), distance-bias attention (32 buckets up to half the window, query temperature, output
+    gate, one more 1 in the denominator) and soft-capped window attention (half of each head rotated) in turn, values
+    mixed across the last two kinds; gated experts of the Mixtral stack's width, 8 + 2 identity outputs in two groups of
+    which the better one is kept, two choices per token, a shared expert of a quarter of the width."""
+    w, ff, d = s["width"], s["ff"], s["dim"]
+    moe = {"kind": "moe", "router": {"experts": 8, "identity": 2, "top": 2, "groups": {"count": 2, "keep": 1}},
+           "expert": {"ff": ff}, "shared": {"ff": ff // 4}}
+    rank, rot = (128, 32) if d <= 64 else (512, 64)
+    lat = {"type": "latent_attention",
+           "mixer": {"heads": s["heads"], "dim": d, "rot_dim": rot, "vdim": d, "kv_rank": rank, "q_rank": w // 2,
+                     "scale": (d + rot) ** -0.5, "rot": {"base": 50000.0, "dims": rot}}}
+    common = {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": d, "vdim": d, "scale": d ** -0.5, "v_mix": True}
+    bias = {"type": "attention", "mixer": dict(common, bias_max=s["window"] // 2, bias_rows=32,
+                                               q_temp={"coef": 0.5, "every": 256})}
+    cap = {"type": "attention_2", "mixer": dict(common, mask={"size": s["window"]}, softcap=30.0,
+                                                rot={"base": 10000.0, "dims": d // 2})}
+    return {"architecture": "Lefolorn", "vocab": s["vocab"], "width": w, "norm": {"eps": 1e-6, "groups": 4},
+            "layers": [dict((lat, bias, cap)[i % 3], mlp=moe) for i in range(s["layers"])]}
+
+
+MODELS = {"lefolorn": lefolorn_config, "sevazen": sevazen_config, "mixtral-swa": mixtral_swa_config, "nositar": nositar_config, "llama-swa": llama_config, "jamba": jamba_config, "jamba-moe": jamba_moe_config,
           "rapovik": rapovik_config}
 
 

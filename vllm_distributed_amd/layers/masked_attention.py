@@ -198,11 +198,13 @@ class MaskedSoftmaxAttention(nn.Module):
 
     def _distances(self) -> Optional[torch.Tensor]:
         """fp32 [far + 1, H]: the bias of every distance, the learned rows spread over their buckets (made once from
-        the loaded table)."""
+        the loaded table); for the matrix-core kernels one padded row per head instead."""
         if not self.dist_far:
             return None
         if self._dist_table is None or self._dist_table.device != self.rel.device:
             self._dist_table = self.rel.data[self._bucket.to(self.rel.device)].contiguous()
+            if self.use_mfma:             # one padded row per head
+                self._dist_table = ops.padded_distance_rows(self._dist_table)
         return self._dist_table
 
     def _lambda(self) -> Optional[torch.Tensor]:

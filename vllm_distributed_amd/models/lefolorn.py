@@ -175,9 +175,9 @@ class LefolornLayer(nn.Module):
         subs = [(y, self.ls1, g[:, :W], None, None)]
         if self.has_mlp:
             f, shared, idw = self.mlp(h)
-            if shared is not None:
-                f = f + shared
             subs.append((f, self.ls2, g[:, W:], h if idw is not None else None, idw))
+            if shared is not None:              # joins inside the same pass, behind the feed-forward's scale and gate
+                subs.append((shared, self.ls2, g[:, W:], None, None))
         return ops.gated_residual_group_norm(x, subs, next_norm, groups, eps, h.dtype)
 
 

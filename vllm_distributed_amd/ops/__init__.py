@@ -249,7 +249,8 @@ def paged_attention_decode(out, q, k_cache, v_cache, block_table, seq_lens, q_st
     """q, out: [T, Hq, D].  Each sequence has <= max_q_len query tokens (1 for plain decode).
     ``sink`` fp32 [Hq]: exp(sink[h]) joins head h's softmax denominator; ``chunk`` > 0: keys of the query's own chunk
     of that many positions only; ``v_shift``: K head k reads V head k >> v_shift (v_cache holds that many fewer heads);
-    ``dist_bias`` fp32 [far + 1, Hq]: row min(query position - key position, far) joins the scores.
+    ``dist_bias`` (rows of ``padded_distance_rows``): the value of min(query position - key position, far) joins head
+    h's scores.
     These four are options of the device kernels only."""
     T, Hq, D = q.shape
     if not _dev(q):
@@ -273,12 +274,24 @@ def paged_attention_decode(out, q, k_cache, v_cache, block_table, seq_lens, q_st
     return out
 
 
+DIST_PAD = 32           # entries before and after a head's distances in the rows of ``padded_distance_rows``
+
+
+def padded_distance_rows(table: torch.Tensor) -> torch.Tensor:
+    """A bias table fp32 [far + 1, Hq] (one row per distance) in the layout the matrix-core attention kernels read:
+    one row per head, [Hq, DIST_PAD + far + 1 + DIST_PAD] -- DIST_PAD zeros (distances below zero belong to masked
+    keys), the head's values, then its last value DIST_PAD times more."""
+    t = table.float().t()
+    return torch.cat([t.new_zeros((t.shape[0], DIST_PAD)), t, t[:, -1:].expand(-1, DIST_PAD)], dim=1).contiguous()
+
+
 def _dist_bias_args(dist_bias: Optional[torch.Tensor], Hq: int) -> tuple:
+    """``dist_bias``: rows of ``padded_distance_rows``."""
     if dist_bias is None:
         return None, 0
     assert dist_bias.dtype == torch.float32 and dist_bias.is_contiguous() and dist_bias.dim() == 2 \
-        and dist_bias.shape[1] == Hq
-    return dist_bias.data_ptr(), dist_bias.shape[0] - 1
+        and dist_bias.shape[0] == Hq and dist_bias.shape[1] > 2 * DIST_PAD
+    return dist_bias.data_ptr(), dist_bias.shape[1] - 2 * DIST_PAD - 1
 
 
 def paged_attention_prefill(out, q, k_cache, v_cache, block_table, seq_lens, q_start_loc, scale: float,
@@ -1564,12 +1577,12 @@ def residual_norms(x: torch.Tensor, y: Optional[torch.Tensor] = None, w_post: Op
 def gated_residual_group_norm(x: torch.Tensor, subs: list, w_next: Optional[torch.Tensor], groups: int, eps: float,
                               out_dtype: torch.dtype) -> Optional[torch.Tensor]:
     """One pass over the fp32 residual ``x`` [T, W]: x += sum over ``subs`` of (y + extra_w[:, None] * extra) * scale *
-    sigmoid(gate), in place -- one tuple (y, scale, gate, extra, extra_w) per sub-layer (at most two; y [T, W] in the
+    sigmoid(gate), in place -- one tuple (y, scale, gate, extra, extra_w) per sub-layer (at most three; y [T, W] in the
     activation type, scale fp32 [W] or None, gate [T, W] pre-activations or None, extra [T, W] with extra_w fp32 [T] or
     None) -- and, with ``w_next`` (fp32 [W]), returns the updated row normalised in ``groups`` equal consecutive parts,
     each divided by its own root mean square, times w_next, in ``out_dtype``."""
     T, W = x.shape
-    if not _dev(x) or (W + groups) * 4 > 60 * 1024 or len(subs) > 2:
+    if not _dev(x) or (W + groups) * 4 > 60 * 1024 or len(subs) > 3:
         return R.gated_residual_group_norm(x, subs, w_next, groups, eps, out_dtype)
     assert x.dtype == torch.float32 and x.is_contiguous() and W % groups == 0
     h = torch.empty((T, W), dtype=out_dtype, device=x.device) if w_next is not None else None
@@ -1585,7 +1598,7 @@ def gated_residual_group_norm(x: torch.Tensor, subs: list, w_next: Optional[torc
                                  and extra_w.dtype == torch.float32 and extra_w.is_contiguous() and extra_w.numel() == T)
         args += [y.data_ptr(), y.stride(0), N.ptr(scale), N.ptr(gate), gate.stride(0) if gate is not None else 0,
                  N.ptr(extra), extra.stride(0) if extra is not None else 0, N.ptr(extra_w)]
-    args += [None, 0, None, None, 0, None, 0, None] * (2 - len(subs))
+    args += [None, 0, None, None, 0, None, 0, None] * (3 - len(subs))
     assert h is None or not subs or h.dtype == dt
     N.call("vda_gated_residual_group_norm", x.data_ptr(), len(subs), *args, N.ptr(w_next), N.ptr(h),
            h.stride(0) if h is not None else 0, float(eps), int(groups), T, W, N.dt(dt), N.stream())

@@ -32,9 +32,32 @@ struct AttnParams {
   const float* sink;        // [Hq]: exp(sink[h]) joins head h's softmax denominator, with no key and no value
   int chunk;                // > 0: the query at position i sees keys j with j / chunk == i / chunk only
   int v_shift;              // K head k reads V head k >> v_shift (the V cache then holds Hkv >> v_shift heads)
-  const float* dist_bias;   // [dist_far + 1, Hq]: row min(query position - key position, dist_far) joins the scores
-  int dist_far;             //   of every head (after the scale and the soft cap)
+  // a bias per (head, query position - key position) joins the scores after the scale and the soft cap; distances from
+  // dist_far on share one value.  One row per head, [Hq][DIST_PAD + dist_far + 1 + DIST_PAD]: DIST_PAD unused entries
+  // (distances below zero: masked keys), the values of distances 0 .. dist_far, then the last value DIST_PAD times
+  // more, so that a lane reads the biases of consecutive keys with one clamped 16-byte load
+  const float* dist_bias;
+  int dist_far;
 };
+
+constexpr int DIST_PAD = 32;
+
+__device__ __forceinline__ const float* dist_row(const AttnParams& p, int head) {
+  return p.dist_bias + (long)head * (p.dist_far + 1 + 2 * DIST_PAD) + DIST_PAD;
+}
+
+// the biases of the four distances d_lo .. d_lo + 3 (a row of dist_row)
+__device__ __forceinline__ f32x4 dist_bias4(const float* row, int d_lo, int far) {
+  f32x4 v;
+  __builtin_memcpy(&v, row + min(max(d_lo, -DIST_PAD), far), 16);      // 4-byte aligned
+  return v;
+}
+
+// tanh through one exponential and one reciprocal: absolute error of a few 1e-7, which a soft cap of some tens turns
+// into 1e-5 of a score at most
+__device__ __forceinline__ float fast_tanh(float x) {
+  return 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + fexp2(x * 2.8853900817779268f));
+}
 
 // Key selection of the sparse prefill form: per (sequence, head) a list of single key positions ("vertical" lines of
 // the score matrix) and a list of query-minus-key distances ("slash" lines), both in absolute positions of the

@@ -80,8 +80,8 @@ __global__ __launch_bounds__(256) void paged_attn_kernel(AttnParams p) {
     if (valid && p.chunk > 0) lower[ct] = max(lower[ct], (limit[ct] - 1) / p.chunk * p.chunk);
     const int head = kvh * G + h;
     slope[ct] = (p.alibi && valid) ? p.alibi[head] : 0.f;
-    bias_col[ct] = p.dist_bias ? p.dist_bias + head : nullptr;
-    bfar2[ct] = (p.dist_bias && valid) ? p.dist_bias[(long)p.dist_far * p.Hq + head] * 1.4426950408889634f : 0.f;
+    bias_col[ct] = p.dist_bias ? dist_row(p, head) : nullptr;
+    bfar2[ct] = (p.dist_bias && valid) ? bias_col[ct][p.dist_far] * 1.4426950408889634f : 0.f;
     // a sink is a score without key or value: the running maximum starts there and the sum with its weight of one
     // (once per column: in the lane group that holds the sum's first part, and in split mode in one wave of one part)
     sink_m[ct] = (p.sink && valid && (!SPLIT || (wave == 0 && blockIdx.z == 0))) ? p.sink[head] * 1.4426950408889634f
@@ -166,13 +166,20 @@ __global__ __launch_bounds__(256) void paged_attn_kernel(AttnParams p) {
       }
       float sv[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
       float mx = -INFINITY;
+      float bj[8] = {0, 0, 0, 0, 0, 0, 0, 0};         // key tb + j sits limit - 1 - tb - j behind the query
+      if (p.dist_bias) {
+        const int d_lo = limit[ct] - 1 - (tb + 7);
+        const f32x4 b0 = dist_bias4(bias_col[ct], d_lo, p.dist_far), b1 = dist_bias4(bias_col[ct], d_lo + 4, p.dist_far);
+        bj[7] = b0[0]; bj[6] = b0[1]; bj[5] = b0[2]; bj[4] = b0[3];
+        bj[3] = b1[0]; bj[2] = b1[1]; bj[1] = b1[2]; bj[0] = b1[3];
+      }
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const int tok = tb + j;
         float x = sv[j] * p.scale;
-        if (p.softcap > 0.f) x = p.softcap * tanhf(x / p.softcap);
+        if (p.softcap > 0.f) x = p.softcap * fast_tanh(x / p.softcap);
         x += slope[ct] * (float)(tok - (limit[ct] - 1));
-        if (p.dist_bias) x += bias_col[ct][(long)min(max(limit[ct] - 1 - tok, 0), p.dist_far) * p.Hq];
+        x += bj[j];
         x *= 1.4426950408889634f;
         x = (tok < limit[ct] && tok >= lower[ct]) ? x : -INFINITY;
         sv[j] = x;
@@ -377,8 +384,8 @@ __global__ __launch_bounds__(256, PREFILL_WGS_PER_CU) void paged_prefill_lds_ker
     if (valid && p.chunk > 0) lower[ct] = max(lower[ct], (limit[ct] - 1) / p.chunk * p.chunk);
     const int head = head0 + h;
     slope[ct] = (p.alibi && valid) ? p.alibi[head] : 0.f;
-    bias_col[ct] = p.dist_bias ? p.dist_bias + head : nullptr;
-    bfar2[ct] = (p.dist_bias && valid) ? p.dist_bias[(long)p.dist_far * p.Hq + head] * 1.4426950408889634f : 0.f;
+    bias_col[ct] = p.dist_bias ? dist_row(p, head) : nullptr;
+    bfar2[ct] = (p.dist_bias && valid) ? bias_col[ct][p.dist_far] * 1.4426950408889634f : 0.f;
     sink_m[ct] = (p.sink && valid) ? p.sink[head] * 1.4426950408889634f : -INFINITY;
     const T* qp = (const T*)p.q + (long)(qs + (valid ? qt : q0)) * p.q_stride + (long)head * D + g * DQ;
 #pragma unroll
@@ -539,17 +546,24 @@ __global__ __launch_bounds__(256, PREFILL_WGS_PER_CU) void paged_prefill_lds_ker
         for (int j = 0; j < 8; ++j) mx = fmaxf(mx, sv[j]);
         mx = fmaf(mx, sl2, bfar2[ct]);
       } else {
+        // a tile at least dist_far behind every column of the wave takes the table's last value throughout
+        float bj[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) bj[j] = bfar2[ct];
+        if (p.dist_bias && !far_tile) {
+          const int d_lo = limit[ct] - 1 - (tb + 7);
+          const f32x4 b0 = dist_bias4(bias_col[ct], d_lo, p.dist_far) * 1.4426950408889634f;
+          const f32x4 b1 = dist_bias4(bias_col[ct], d_lo + 4, p.dist_far) * 1.4426950408889634f;
+          bj[7] = b0[0]; bj[6] = b0[1]; bj[5] = b0[2]; bj[4] = b0[3];
+          bj[3] = b1[0]; bj[2] = b1[1]; bj[1] = b1[2]; bj[0] = b1[3];
+        }
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const int tok = tb + j;
           float x = sv[j] * p.scale;
-          if (p.softcap > 0.f) x = p.softcap * tanhf(x / p.softcap);
+          if (p.softcap > 0.f) x = p.softcap * fast_tanh(x / p.softcap);
           x += slope[ct] * (float)(tok - (limit[ct] - 1));
-          x *= 1.4426950408889634f;
-          // a tile at least dist_far behind every column of the wave takes the table's last row throughout
-          if (p.dist_bias)
-            x += far_tile ? bfar2[ct] : 1.4426950408889634f *
-                 bias_col[ct][(long)min(max(limit[ct] - 1 - tok, 0), p.dist_far) * p.Hq];
+          x = fmaf(x, 1.4426950408889634f, bj[j]);
           x = (tok < limit[ct] && tok >= lower[ct]) ? x : -INFINITY;
           sv[j] = x;
           mx = fmaxf(mx, x);

@@ -126,7 +126,8 @@ __global__ __launch_bounds__(512) void paged_prefill_wide_kernel(AttnParams p, i
   int lower = (valid && p.window > 0) ? max(0, limit - p.window) : 0;
   if (valid && p.chunk > 0) lower = max(lower, (limit - 1) / p.chunk * p.chunk);     // keys of the query's chunk only
   const float slope = (p.alibi && valid) ? p.alibi[head] : 0.f;
-  const float* bias_col = p.dist_bias ? p.dist_bias + head : nullptr;      // this column's distance biases
+  const float* bias_col = p.dist_bias ? dist_row(p, head) : nullptr;       // this column's distance biases
+  const float bfar2 = (p.dist_bias && valid) ? bias_col[p.dist_far] * 1.4426950408889634f : 0.f;
   const long col_off = valid ? (long)(qs + qt) : -1;
   V8 qf[8];
   {
@@ -223,6 +224,7 @@ __global__ __launch_bounds__(512) void paged_prefill_wide_kernel(AttnParams p, i
     for (int r = 0; r < 16; ++r) acc[db][r] = 0.f;
 
   const float sl2 = p.scale * 1.4426950408889634f;
+  const bool far_plain = p.dist_bias != nullptr && !(p.softcap > 0.f) && p.alibi == nullptr;
 
   // A tile is worked in two halves of 32 keys, each with its own online-softmax update, ordered so that the
   // vector ALU and the matrix pipe have independent work inside one wave:
@@ -244,16 +246,25 @@ __global__ __launch_bounds__(512) void paged_prefill_wide_kernel(AttnParams p, i
   auto softmax_half = [&](int tb, int kb, V8 (&pb)[2], auto mode) -> float {
     constexpr int MODE = decltype(mode)::value;
     float mx = -INFINITY;
+    f32x4 bq[4];                                   // MODE 2: the biases of this lane's four runs of four keys
+    if constexpr (MODE == 2) {
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        bq[q4] = f32x4{0, 0, 0, 0};
+        // keys tb + 8 q4 + 4 hi + (0 .. 3) sit limit - 1 - key behind the query: ascending distances from the last
+        if (bias_col) bq[q4] = dist_bias4(bias_col, limit - 1 - (tb + 8 * q4 + 4 * hi + 3), p.dist_far);
+      }
+    }
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       float x = S[kb][r];
-      if constexpr (MODE >= 1) {
+      if constexpr (MODE == 1 || MODE == 2) {
         const int tok = tb + (r & 3) + 8 * (r >> 2) + 4 * hi;
         if constexpr (MODE == 2) {
           x *= p.scale;
-          if (p.softcap > 0.f) x = p.softcap * tanhf(x / p.softcap);
+          if (p.softcap > 0.f) x = p.softcap * fast_tanh(x / p.softcap);
           x += slope * (float)(tok - (limit - 1));
-          if (bias_col) x += bias_col[(long)min(max(limit - 1 - tok, 0), p.dist_far) * p.Hq];
+          x += bq[r >> 2][3 - (r & 3)];
           x *= 1.4426950408889634f;
         }
         x = (tok < limit && tok >= lower) ? x : -INFINITY;
@@ -261,19 +272,24 @@ __global__ __launch_bounds__(512) void paged_prefill_wide_kernel(AttnParams p, i
       }
       mx = fmaxf(mx, x);
     }
+    // MODE 3: an unmasked tile at least dist_far behind every column, no soft cap, no ALiBi: the table's last value
+    // joins the exponent's fma as a constant
     const float mul = MODE == 2 ? 1.f : sl2;
-    if constexpr (MODE != 2) mx *= sl2;          // the scale is positive
+    float off = -INFINITY;
+    if constexpr (MODE == 3) mx = fmaf(mx, sl2, bfar2);
+    else if constexpr (MODE != 2) mx *= sl2;          // the scale is positive
     mx = pair_max(mx);
     const float m_new = fmaxf(m, mx);
     const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
     const float alpha = fexp2(m - m_use);
     m = m_new;
+    off = MODE == 3 ? bfar2 - m_use : -m_use;
     float ps = 0.f;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const float e = fexp2(fmaf(S[kb][8 * t + j], mul, -m_use));
+        const float e = fexp2(fmaf(S[kb][8 * t + j], mul, off));
         ps += e;
         pb[t][j] = (T)e;
       }
@@ -370,7 +386,10 @@ __global__ __launch_bounds__(512) void paged_prefill_wide_kernel(AttnParams p, i
 #endif
     } else {
       if constexpr (GENERAL) {
-        tile_compute(kt, buf, std::integral_constant<int, 2>{});
+        if (far_plain && tb0 + KT <= full_hi - p.dist_far && tb0 >= full_lo)
+          tile_compute(kt, buf, std::integral_constant<int, 3>{});
+        else
+          tile_compute(kt, buf, std::integral_constant<int, 2>{});
       } else {
         if (tb0 + KT <= full_hi && tb0 >= full_lo) tile_compute(kt, buf, std::integral_constant<int, 0>{});
         else tile_compute(kt, buf, std::integral_constant<int, 1>{});

@@ -297,7 +297,8 @@ VDA_EXPORT int vda_group_rms_norm(void* out, long o_stride, const void* x, long 
 //   x[t] += sum over the sub-layers of (y + extra_w[t] * extra) * scale * sigmoid(gate)      (in place, fp32)
 //   h[t]  = x[t] / rms_g(x[t]) * w_next    with rms_g the root mean square of the value's own part, the row being
 //           split into `groups` equal consecutive parts
-// Every piece is optional: no sub-layer at all is the stack's first or last norm, no h is the last residual update.
+// Every piece is optional: no sub-layer at all is the stack's first or last norm, no h is the last residual update; up to
+// three sub-layer outputs join in one pass (a shared expert beside the routed ones takes the third place).
 // One workgroup per token; the updated row waits in LDS for its parts' sums.
 struct GatedSub {
   const void* y;        // [T, W] the sub-layer's output
@@ -311,7 +312,7 @@ struct GatedSub {
 };
 struct GatedResidualArgs {
   float* x;
-  GatedSub sub[2];
+  GatedSub sub[3];
   int nsub;
   const float* w_next;
   void* h;
@@ -383,11 +384,12 @@ __global__ __launch_bounds__(256) void gated_residual_group_norm_kernel(const Ga
 VDA_EXPORT int vda_gated_residual_group_norm(
     float* x, int nsub, const void* y0, long y0_stride, const float* s0, const void* g0, long g0_stride,
     const void* e0, long e0_stride, const float* ew0, const void* y1, long y1_stride, const float* s1, const void* g1,
-    long g1_stride, const void* e1, long e1_stride, const float* ew1, const float* w_next, void* h, long h_stride,
-    float eps, int groups, int T, int W, int dtype, hipStream_t st) {
+    long g1_stride, const void* e1, long e1_stride, const float* ew1, const void* y2, long y2_stride, const float* s2,
+    const void* g2, long g2_stride, const void* e2, long e2_stride, const float* ew2, const float* w_next, void* h,
+    long h_stride, float eps, int groups, int T, int W, int dtype, hipStream_t st) {
   if (T <= 0 || (nsub == 0 && !h)) return 0;
-  if (nsub < 0 || nsub > 2 || (nsub > 0 && !y0) || (nsub > 1 && !y1) || (h && !w_next) || groups < 1 || W % groups ||
-      (e0 && !ew0) || (e1 && !ew1))
+  if (nsub < 0 || nsub > 3 || (nsub > 0 && !y0) || (nsub > 1 && !y1) || (nsub > 2 && !y2) || (h && !w_next) ||
+      groups < 1 || W % groups || (e0 && !ew0) || (e1 && !ew1) || (e2 && !ew2))
     return -1;
   const size_t lds = ((size_t)W + groups) * 4;
   if (lds > 60 * 1024) return -2;
@@ -395,6 +397,7 @@ VDA_EXPORT int vda_gated_residual_group_norm(
   a.x = x; a.nsub = nsub; a.w_next = w_next; a.h = h; a.h_stride = h_stride; a.eps = eps; a.W = W; a.groups = groups;
   a.sub[0] = GatedSub{y0, y0_stride, s0, g0, g0_stride, e0, e0_stride, ew0};
   a.sub[1] = GatedSub{y1, y1_stride, s1, g1, g1_stride, e1, e1_stride, ew1};
+  a.sub[2] = GatedSub{y2, y2_stride, s2, g2, g2_stride, e2, e2_stride, ew2};
   bool vec = W % 4 == 0 && h_stride % 4 == 0;
   for (int i = 0; i < nsub; ++i)
     vec = vec && a.sub[i].y_stride % 4 == 0 && a.sub[i].gate_stride % 4 == 0 && a.sub[i].extra_stride % 4 == 0;

@@ -65,7 +65,7 @@ _SIGS = {
     "vda_mlstm": [P, L, P, P, L, P, P, P, P, P, P, P, P, L, I, I, I, I, I, I, F, F, I, P],
     "vda_moe_grouped_sigmoid_topk": [P, P, P, P, I, I, I, I, I, I, L, I, P],
     "vda_moe_grouped_topk": [P, P, P, P, P, I, I, I, I, I, I, F, I, I, I, L, I, P],
-    "vda_gated_residual_group_norm": [P, I, P, L, P, P, L, P, L, P, P, L, P, P, L, P, L, P, P, P, L, F, I, I, I, I, P],
+    "vda_gated_residual_group_norm": [P, I] + [P, L, P, P, L, P, L, P] * 3 + [P, P, L, F, I, I, I, I, P],
     "vda_group_rms_norm": [P, L, P, L, P, F, I, I, I, I, I, P],
     "vda_moe_pairs": [P, L, P, P, L, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
     "vda_residual_layer_norm": [P, P, L, P, P, P, L, F, I, I, I, P, L, P, L, P],
