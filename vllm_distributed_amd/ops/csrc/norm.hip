@@ -381,6 +381,87 @@ __global__ __launch_bounds__(256) void gated_residual_group_norm_kernel(const Ga
   }
 }
 
+// The same with the row in registers: TRIPS trips of 256 * 4 values cover it, and every wave's 256 values of a trip
+// lie inside one part (part % 256 == 0), so a part's sum of squares is the sum of whole-wave sums, added up in a fixed
+// order by every thread for its own parts.  One barrier, no pass through LDS for the row.
+template <typename T, int TRIPS>
+__global__ __launch_bounds__(256) void gated_residual_group_norm_reg_kernel(const GatedResidualArgs a) {
+  __shared__ float wsum[TRIPS * 4];
+  const long t = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int W = a.W;
+  float* xr = a.x + t * W;
+  float v[TRIPS][4];
+#pragma unroll
+  for (int k = 0; k < TRIPS; ++k) {
+    const int c = (k * 256 + tid) * 4;
+    const bool live = c < W;
+    float add[4] = {0.f, 0.f, 0.f, 0.f};
+    if (live) {
+      const f32x4 q = *reinterpret_cast<const f32x4*>(xr + c);
+      v[k][0] = q[0]; v[k][1] = q[1]; v[k][2] = q[2]; v[k][3] = q[3];
+      for (int sI = 0; sI < a.nsub; ++sI) {
+        const GatedSub& u = a.sub[sI];
+        using V4 = typename Vec<T>::v4;
+        const V4 y4 = *reinterpret_cast<const V4*>((const T*)u.y + t * u.y_stride + c);
+        float f[4] = {(float)y4[0], (float)y4[1], (float)y4[2], (float)y4[3]};
+        if (u.extra) {
+          const V4 e4 = *reinterpret_cast<const V4*>((const T*)u.extra + t * u.extra_stride + c);
+          const float ew = u.extra_w[t];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) f[i] += ew * (float)e4[i];
+        }
+        if (u.scale) {
+          const f32x4 s4 = *reinterpret_cast<const f32x4*>(u.scale + c);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) f[i] *= s4[i];
+        }
+        if (u.gate) {
+          const V4 g4 = *reinterpret_cast<const V4*>((const T*)u.gate + t * u.gate_stride + c);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) f[i] *= 1.f / (1.f + expf(-(float)g4[i]));
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) add[i] += f[i];
+      }
+      if (a.nsub > 0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[k][i] += add[i];
+        *reinterpret_cast<f32x4*>(xr + c) = f32x4{v[k][0], v[k][1], v[k][2], v[k][3]};
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[k][i] = 0.f;
+    }
+    if (a.h) {
+      float ss = v[k][0] * v[k][0] + v[k][1] * v[k][1] + v[k][2] * v[k][2] + v[k][3] * v[k][3];
+      ss = wave_sum(ss);
+      if (lane == 0) wsum[k * 4 + wave] = ss;
+    }
+  }
+  if (!a.h) return;
+  __syncthreads();
+  const int part = W / a.groups;
+  T* hr = (T*)a.h + t * a.h_stride;
+#pragma unroll
+  for (int k = 0; k < TRIPS; ++k) {
+    const int c = (k * 256 + tid) * 4;
+    if (c >= W) continue;
+    const int g = c / part;
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < TRIPS * 4; ++j)               // chunk j holds the values from j * 256 on
+      if ((j * 256) / part == g) ss += wsum[j];
+    const float r = 1.f / sqrtf(ss / (float)part + a.eps);
+    const f32x4 w4 = *reinterpret_cast<const f32x4*>(a.w_next + c);
+    using V4 = typename Vec<T>::v4;
+    V4 o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = (T)(v[k][i] * r * w4[i]);
+    *reinterpret_cast<V4*>(hr + c) = o;
+  }
+}
+
 VDA_EXPORT int vda_gated_residual_group_norm(
     float* x, int nsub, const void* y0, long y0_stride, const float* s0, const void* g0, long g0_stride,
     const void* e0, long e0_stride, const float* ew0, const void* y1, long y1_stride, const float* s1, const void* g1,
@@ -401,14 +482,33 @@ VDA_EXPORT int vda_gated_residual_group_norm(
   bool vec = W % 4 == 0 && h_stride % 4 == 0;
   for (int i = 0; i < nsub; ++i)
     vec = vec && a.sub[i].y_stride % 4 == 0 && a.sub[i].gate_stride % 4 == 0 && a.sub[i].extra_stride % 4 == 0;
+  // rows of up to 4096 values whose parts are whole numbers of 256-value wave chunks stay in registers
+  const int trips = (W + 1023) / 1024;
+  const uintptr_t al = dtype == VDA_F32 ? 16 : 8;          // four values of the activation type
+  const bool reg = vec && trips <= 4 && (W / groups) % 256 == 0 && ((uintptr_t)x % 16 == 0) &&
+                   (!w_next || (uintptr_t)w_next % 16 == 0) && (!h || (uintptr_t)h % al == 0) && [&] {
+                     for (int i = 0; i < nsub; ++i) {
+                       const GatedSub& u = a.sub[i];
+                       if ((uintptr_t)u.y % al || (uintptr_t)u.gate % al || (uintptr_t)u.extra % al ||
+                           (uintptr_t)u.scale % 16)
+                         return false;
+                     }
+                     return true;
+                   }();
+#define LR(TT, KK) hipLaunchKernelGGL((gated_residual_group_norm_reg_kernel<TT, KK>), dim3(T), dim3(256), 0, st, a)
 #define L2(TT, VV) hipLaunchKernelGGL((gated_residual_group_norm_kernel<TT, VV>), dim3(T), dim3(256), lds, st, a)
-#define L(TT) do { if (vec) L2(TT, 4); else L2(TT, 1); } while (0)
+#define L(TT)                                                                                                       \
+  do {                                                                                                              \
+    if (reg && trips == 1) LR(TT, 1); else if (reg && trips == 2) LR(TT, 2); else if (reg && trips == 3) LR(TT, 3); \
+    else if (reg) LR(TT, 4); else if (vec) L2(TT, 4); else L2(TT, 1);                                               \
+  } while (0)
   if (dtype == VDA_BF16) L(bf16_t);
   else if (dtype == VDA_F16) L(f16_t);
   else if (dtype == VDA_F32) L(float);
   else return -3;
 #undef L
 #undef L2
+#undef LR
   VDA_CHECK_LAUNCH();
   return 0;
 }
