@@ -553,6 +553,20 @@ def test_a_tensor_without_a_place_is_refused(tmp_path):
         TraceReplayer(folder, "float32", 64, device="cpu", enforce_eager=True)
 
 
+def test_tensors_the_design_never_reads_are_skipped(tmp_path):
+    """A checkpoint may carry the feed-forward's scale and gate for a layer that has none, and a mixing weight for the
+    layer that lends its values: they change nothing."""
+    cfg = O.make_config([O.cap_layer(v_mix=True, mlp=None), O.bias_layer(v_mix=True, mlp=None)])
+    W = O.make_weights(cfg, 0)
+    p = tokens(9, cfg["vocab"], 1)
+    want = O.forward(cfg, W, p)
+    W["l0.ls2"], W["l0.rg2"], W["l0.rg2.b"] = W["l0.ls1"].clone(), W["l0.rg1"].clone(), W["l0.rg1.b"].clone()
+    W["l0.mix.vmix"] = torch.tensor(0.9, dtype=torch.bfloat16)
+    folder = O.save_checkpoint(str(tmp_path / "m"), cfg, W)
+    got = run_schedule(folder, "float32", "cpu", {"a": p}, [[("a", 9)]], 16)
+    assert O.logit_error(got["a"], want) < TOL["float32"]
+
+
 @pytest.mark.parametrize("dev,dtype", CASES)
 @pytest.mark.parametrize("layers", list(LAYER_SETS))
 def test_prefill_equals_decoding_token_by_token(tmp_path, dev, dtype, layers):

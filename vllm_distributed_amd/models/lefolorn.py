@@ -242,6 +242,7 @@ class LefolornForCausalLM(nn.Module):
     _EXPERT = {"gate": ("w13_weight", "w1"), "up": ("w13_weight", "w3"), "down": ("w2_weight", "w2")}
     _LAYER = {"norm1": ("norm1", None), "ls1": ("ls1", None), "ls2": ("ls2", None), "rg1": ("gates.weight", 0),
               "rg1.b": ("gates.bias", 0), "rg2": ("gates.weight", 1), "rg2.b": ("gates.bias", 1)}
+    _FF_ONLY = ("ls2", "rg2", "rg2.b")
 
     def _target(self, name: str):
         """Returns (parameter name, shard id, expert id) or None."""
@@ -254,6 +255,8 @@ class LefolornForCausalLM(nn.Module):
         layer, base = self.layers[i], f"layers.{i}."
         if rest in self._LAYER:
             t, shard = self._LAYER[rest]
+            if rest in self._FF_ONLY and not layer.has_mlp:
+                return base + "no_feed_forward." + rest, None, None
             return base + t, shard, None
         part, _, leaf = rest.partition(".")
         if part == "mix" and leaf in self._MIX[layer.kind]:
@@ -283,9 +286,9 @@ class LefolornForCausalLM(nn.Module):
                 raise ValueError(f"checkpoint tensor {name!r} has no place in this model")
             target, shard, expert = tgt
             if target not in params:
-                # the value-mixing weight of the first layer that mixes is never used; a layer that does not mix
-                # has no place for one
-                if name.endswith(".mix.vmix"):
+                # tensors the design never reads: the value-mixing weight of a layer that lends its values or does not
+                # mix, the feed-forward's scale and gate of a layer without a feed-forward
+                if name.endswith((".mix.vmix", ".ls2", ".rg2", ".rg2.b")):
                     continue
                 raise ValueError(f"checkpoint tensor {name!r} has no place in this model")
             p = params[target]
