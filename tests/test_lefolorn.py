@@ -197,10 +197,11 @@ def test_group_limited_softmax_choice_with_identity_outputs(dev, dt, n, ident, t
 
 @pytest.mark.parametrize("dev,dt", OP_CASES)
 @pytest.mark.parametrize("Wd,ff,E,ident,top,T", [(24, 10, 5, 1, 2, 9), (33, 7, 3, 2, 3, 4), (48, 80, 6, 0, 3, 70),
-                                                 (256, 128, 8, 2, 2, 150), (128, 64, 4, 4, 2, 3)])
+                                                 (256, 128, 8, 2, 2, 150), (128, 64, 4, 4, 2, 3),
+                                                 (256, 128, 8, 2, 2, 1300)])
 def test_gated_experts_with_identity_choices(dev, dt, Wd, ff, E, ident, top, T):
     """The experts' weighted sum when some winners have no expert (their share is the input itself); the last sizes are
-    ones the matrix-core expert kernels take in 16-bit."""
+    ones the matrix-core expert kernels take in 16-bit (few pairs: the grouped skinny form, many: the tiled form)."""
     from vllm_distributed_amd.layers.moe import grouped_topk_with_identity
     x = torch.randn(T, Wd).to(dt)
     n = E + ident
