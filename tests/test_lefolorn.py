@@ -124,7 +124,7 @@ def pages(lens, bs, spare=3):
 # ---- mechanisms alone ----------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dev,dt", OP_CASES)
 @pytest.mark.parametrize("W_,groups", [(48, 4), (300, 3), (33, 1), (512, 8), (70, 7), (512, 2), (1024, 4), (3072, 3),
-                                       (4096, 2), (1280, 5)])
+                                       (4096, 2), (1280, 5), (1024, 8), (2048, 64), (64, 4), (1536, 12)])
 def test_gated_parallel_residual_with_group_norm(dev, dt, W_, groups):
     T, eps = 7, 1e-5
     x = torch.randn(T, W_) * 3 + 1

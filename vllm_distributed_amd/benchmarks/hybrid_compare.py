@@ -145,13 +145,13 @@ def lefolorn_config(s: dict) -> dict:
     rank, rot = (128, 32) if d <= 64 else (512, 64)
     lat = {"type": "latent_attention",
            "mixer": {"heads": s["heads"], "dim": d, "rot_dim": rot, "vdim": d, "kv_rank": rank, "q_rank": w // 2,
-                     "scale": (d + rot) ** -0.5, "rot": {"base": 50000.0, "dims": rot}}}
+                     "scale": (d + rot) ** -0.5, "rot": {"base": 10000.0, "dims": rot}}}
     common = {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": d, "vdim": d, "scale": d ** -0.5, "v_mix": True}
     bias = {"type": "attention", "mixer": dict(common, bias_max=s["window"] // 2, bias_rows=32,
-                                               q_temp={"coef": 0.5, "every": 256})}
+                                               q_temp={"coef": 0.25, "every": 512})}
     cap = {"type": "attention_2", "mixer": dict(common, mask={"size": s["window"]}, softcap=30.0,
                                                 rot={"base": 10000.0, "dims": d // 2})}
-    return {"architecture": "Lefolorn", "vocab": s["vocab"], "width": w, "norm": {"eps": 1e-6, "groups": 4},
+    return {"architecture": "Lefolorn", "vocab": s["vocab"], "width": w, "norm": {"eps": 1e-6, "groups": 8},
             "layers": [dict((lat, bias, cap)[i % 3], mlp=moe) for i in range(s["layers"])]}
 
 

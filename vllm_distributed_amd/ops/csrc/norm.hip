@@ -381,12 +381,16 @@ __global__ __launch_bounds__(256) void gated_residual_group_norm_kernel(const Ga
   }
 }
 
-// The same with the row in registers: TRIPS trips of 256 * 4 values cover it, and every wave's 256 values of a trip
-// lie inside one part (part % 256 == 0), so a part's sum of squares is the sum of whole-wave sums, added up in a fixed
-// order by every thread for its own parts.  One barrier, no pass through LDS for the row.
+// The same with the row in registers: TRIPS trips of 256 * 4 values cover it.  Either every wave's 256 values of a trip
+// lie inside one part (part % 256 == 0): a part's sum of squares is then the sum of whole-wave sums, added up in a
+// fixed order by every thread for its own parts (one barrier, no pass through LDS for the row); or a part is 4 * seg
+// values for a power of two seg <= 64, i.e. seg neighbouring lanes: its sum comes from shuffles alone.
 template <typename T, int TRIPS>
-__global__ __launch_bounds__(256) void gated_residual_group_norm_reg_kernel(const GatedResidualArgs a) {
+__global__ __launch_bounds__(256) void gated_residual_group_norm_reg_kernel(const GatedResidualArgs a, const int seg) {
   __shared__ float wsum[TRIPS * 4];
+  float psum[TRIPS];
+#pragma unroll
+  for (int k = 0; k < TRIPS; ++k) psum[k] = 0.f;
   const long t = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int W = a.W;
@@ -435,23 +439,31 @@ __global__ __launch_bounds__(256) void gated_residual_group_norm_reg_kernel(cons
     }
     if (a.h) {
       float ss = v[k][0] * v[k][0] + v[k][1] * v[k][1] + v[k][2] * v[k][2] + v[k][3] * v[k][3];
-      ss = wave_sum(ss);
-      if (lane == 0) wsum[k * 4 + wave] = ss;
+      if (seg) {                                      // a part is `seg` neighbouring lanes: its sum stays in the wave
+        for (int o = seg >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+        psum[k] = ss;
+      } else {
+        ss = wave_sum(ss);
+        if (lane == 0) wsum[k * 4 + wave] = ss;
+      }
     }
   }
   if (!a.h) return;
-  __syncthreads();
+  if (!seg) __syncthreads();
   const int part = W / a.groups;
   T* hr = (T*)a.h + t * a.h_stride;
 #pragma unroll
   for (int k = 0; k < TRIPS; ++k) {
     const int c = (k * 256 + tid) * 4;
     if (c >= W) continue;
-    const int g = c / part;
-    float ss = 0.f;
+    float ss = psum[k];
+    if (!seg) {
+      const int g = c / part;
+      ss = 0.f;
 #pragma unroll
-    for (int j = 0; j < TRIPS * 4; ++j)               // chunk j holds the values from j * 256 on
-      if ((j * 256) / part == g) ss += wsum[j];
+      for (int j = 0; j < TRIPS * 4; ++j)             // chunk j holds the values from j * 256 on
+        if ((j * 256) / part == g) ss += wsum[j];
+    }
     const float r = 1.f / sqrtf(ss / (float)part + a.eps);
     const f32x4 w4 = *reinterpret_cast<const f32x4*>(a.w_next + c);
     using V4 = typename Vec<T>::v4;
@@ -485,7 +497,10 @@ VDA_EXPORT int vda_gated_residual_group_norm(
   // rows of up to 4096 values whose parts are whole numbers of 256-value wave chunks stay in registers
   const int trips = (W + 1023) / 1024;
   const uintptr_t al = dtype == VDA_F32 ? 16 : 8;          // four values of the activation type
-  const bool reg = vec && trips <= 4 && (W / groups) % 256 == 0 && ((uintptr_t)x % 16 == 0) &&
+  const int part = W / groups;
+  int seg = 0;                                             // lanes per part when a part is a power of two <= 256
+  if (part % 256 != 0 && part >= 4 && part <= 256 && (part & (part - 1)) == 0) seg = part / 4;
+  const bool reg = vec && trips <= 4 && (part % 256 == 0 || seg) && ((uintptr_t)x % 16 == 0) &&
                    (!w_next || (uintptr_t)w_next % 16 == 0) && (!h || (uintptr_t)h % al == 0) && [&] {
                      for (int i = 0; i < nsub; ++i) {
                        const GatedSub& u = a.sub[i];
@@ -495,7 +510,7 @@ VDA_EXPORT int vda_gated_residual_group_norm(
                      }
                      return true;
                    }();
-#define LR(TT, KK) hipLaunchKernelGGL((gated_residual_group_norm_reg_kernel<TT, KK>), dim3(T), dim3(256), 0, st, a)
+#define LR(TT, KK) hipLaunchKernelGGL((gated_residual_group_norm_reg_kernel<TT, KK>), dim3(T), dim3(256), 0, st, a, seg)
 #define L2(TT, VV) hipLaunchKernelGGL((gated_residual_group_norm_kernel<TT, VV>), dim3(T), dim3(256), lds, st, a)
 #define L(TT)                                                                                                       \
   do {                                                                                                              \
