@@ -203,6 +203,8 @@ def test_gated_experts_with_identity_choices(dev, dt, Wd, ff, E, ident, top, T):
     """The experts' weighted sum when some winners have no expert (their share is the input itself); the last sizes are
     ones the matrix-core expert kernels take in 16-bit (few pairs: the grouped skinny form, many: the tiled form)."""
     from vllm_distributed_amd.layers.moe import grouped_topk_with_identity
+    if T > 1000 and dev == "cpu":
+        pytest.skip("the tiled form is a device kernel")
     x = torch.randn(T, Wd).to(dt)
     n = E + ident
     w = {"router": torch.randn(n, Wd) / Wd ** 0.5 * 3, "correction": 0.05 * torch.randn(n)}
