@@ -331,7 +331,7 @@ __global__ __launch_bounds__(512) void paged_prefill_wide_kernel(AttnParams p, i
     // scheduler is told the interleave: one MFMA, then a slice of the softmax.
     auto pin = [](V8 (&pb)[2]) { asm volatile("" : "+v"(pb[0]), "+v"(pb[1])); };
     auto interleave = [] {
-      if constexpr (MODE == 0) {
+      if constexpr (MODE == 0 || MODE == 3) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);     // MFMA
@@ -340,7 +340,7 @@ __global__ __launch_bounds__(512) void paged_prefill_wide_kernel(AttnParams p, i
       }
     };
     qk_half(buf, 0);
-    if constexpr (MODE == 0) __builtin_amdgcn_sched_barrier(0);
+    if constexpr (MODE == 0 || MODE == 3) __builtin_amdgcn_sched_barrier(0);
     if (second) qk_half(buf, 1);
 #if PW_GLOAD_LATE
     issue_next(kt);
