@@ -556,6 +556,20 @@ def test_a_tensor_without_a_place_is_refused(tmp_path):
         TraceReplayer(folder, "float32", 64, device="cpu", enforce_eager=True)
 
 
+def test_benchmark_configurations_are_complete():
+    """The stacks of ``bench.py --compare-lefolorn`` carry every size the model reads, the bucket count included (no
+    checkpoint is there to tell it)."""
+    from vllm_distributed_amd.benchmarks.hybrid_compare import SIZES, lefolorn_config
+    from vllm_distributed_amd.models.lefolorn import normalise_config
+    for size in SIZES.values():
+        d = normalise_config(lefolorn_config(size))
+        assert d["architectures"] == ["LefolornForCausalLM"] and d["num_hidden_layers"] == size["layers"]
+        kinds = {l["type"] for l in d["layers"]}
+        assert kinds == {"latent_attention", "attention", "attention_2"}
+        assert all(l["mixer"]["bias_rows"] >= 2 for l in d["layers"] if l["type"] == "attention")
+        assert d["width"] % d["norm"]["groups"] == 0
+
+
 def test_tensors_the_design_never_reads_are_skipped(tmp_path):
     """A checkpoint may carry the feed-forward's scale and gate for a layer that has none, and a mixing weight for the
     layer that lends its values: they change nothing."""
